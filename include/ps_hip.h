@@ -311,15 +311,18 @@ enum ps_mixer_kind {
     PS_MIX_WINATTN = 4, /* grouped-query attention over a sliding window + one mean key / value per block of `pool` tokens wholly before it,
                          * a sink in the soft-max denominator, a temperature per head, norms over the whole q / k projections, partial rotary, a gate per head */
     PS_MIX_GLA    = 5, /* gated linear attention: S <- diag(alpha) S + k v^T, o = S^T q, a decay per key channel from a two-matrix projection */
+    PS_MIX_MINGRU = 6, /* element-wise gated recurrence, its gates functions of the present input alone: S <- (1 - z) S + z c, output S * silu(g) */
 };
 enum ps_ff_kind {
     PS_FF_NONE = 0,
     PS_FF_DENSE_XIELU = 1,  /* W_down xIELU(W_up h) */
     PS_FF_DENSE_SWIGLU = 2, /* W_down (silu(W_gate h) * (W_up h)); ff_up holds the rows of gate and up INTERLEAVED (gate_0, up_0, gate_1, ...): [2 ff, width] */
+    PS_FF_MOE_SWIGLU = 3,   /* `experts` feed-forwards of the SWIGLU form of which a token uses `top` (fields below), plus an optional shared one */
 };
 enum ps_layer_form {
     PS_LAYER_SEQUENTIAL = 0, /* x += norm_b(mixer(conv(norm1(x)))), then x += norm_b(ff(conv(norm2(x)))) */
-    PS_LAYER_PARALLEL   = 1, /* h = norm1(x); x += mixer(conv(h)) + ff(h): one norm, no norm behind the sublayers, only the mixer's input is filtered */
+    PS_LAYER_PARALLEL   = 1, /* h = norm1(x); x += res_scale (mixer(conv(h)) + ff(h2)): no norm behind the sublayers, only the mixer's input is filtered (canon1 NULL:
+                              * not at all); h2 = h, or norm2(x) where norm2 is given (two weights over the same statistics) */
 };
 enum ps_rot_pairing { PS_ROT_HALVES = 0 /* (i, i + dims/2) */, PS_ROT_NEIGHBOURS = 1 /* (2i, 2i + 1) */ };
 
@@ -372,6 +375,24 @@ typedef struct ps_seq_layer_s {
      *   in_cat = rows of q | k | v | g | a1  ([2*heads*dim + 2*heads*vdim + decay_rank, width]); decay2 [heads*dim, decay_rank]; decay0 [heads*dim] its bias;
      *   alpha = sigmoid(z)^(1/tau), q is scaled by dim^-1/2, the output is per-head RMS-normed (onorm shared by the heads) and multiplied by silu(g) */
     float tau;
+    /* ---- parallel layers */
+    float res_scale;                    /* the sublayers' sum is multiplied by this as it joins the residual stream (0 is taken as 1) */
+    const float *depth_mix;             /* [run + 2] or NULL.  With X_0 the embedding and X_(j+1) the result of layer run j, what leaves run i is
+                                         * sum_j depth_mix[j] X_j over j = 0 .. i + 1 instead of X_(i+1) (parallel layers without an input filter, no loop) */
+    /* ---- attention extras (PS_MIX_WINATTN) */
+    float softcap;                      /* score <- softcap * tanh(score / softcap) after the scale (0: none) */
+    float qtemp_coef;                   /* the query at position p is multiplied by 1 + qtemp_coef * ln(floor((p + 1) / qtemp_every) + 1) (qtemp_every 0: none) */
+    int32_t qtemp_every;
+    /* ---- PS_MIX_MINGRU; it reads dim (the recurrence's width; heads = 1), in_cat = rows of z | x | g ([3 dim, width]), in_bias [3 dim] or NULL, out [width, dim]:
+     *   z = sigmoid(.), c = sigmoid(x) for negative x, else x + 0.5, S <- (1 - z) S + z c element by element (fp32 state, zero at the start), output out (S * silu(g)) */
+    /* ---- PS_FF_MOE_SWIGLU.  router [experts][width] and shared_gate [width] are fp32 vectors: scores = sigmoid(router h) in fp32, the `top` largest are taken
+     * (ties: the lower index), a chosen expert's score multiplies its INPUT (moe_norm_top != 0: the chosen scores are first divided by their sum);
+     *   ff_up   [experts * 2 ff, width]: expert after expert, each with its gate / up rows interleaved;  ff_down [experts * width, ff]
+     *   shared_up [2 shared_ff, width] (interleaved), shared_down [width, shared_ff] or NULL: a feed-forward every token passes, its output times
+     *   sigmoid(shared_gate . h) where shared_gate is given */
+    int32_t experts, top, shared_ff, moe_norm_top;
+    const float *router, *shared_gate;
+    const ps_dense *shared_up, *shared_down;
 } ps_seq_layer;
 
 typedef struct {
@@ -387,7 +408,8 @@ typedef struct {
     /* layers loop_start .. loop_stop - 1 run loop_times times in a row with the same weights, each pass with a state of its own; then the rest follow
      * (loop_times <= 1: every layer runs once).  A "layer run" below is one execution of a layer. */
     int32_t loop_start, loop_stop, loop_times;
-    int32_t max_context; /* most tokens a sequence may hold: sizes what grows with a sequence (the pooled blocks of PS_MIX_WINATTN); 0: 65536 */
+    int32_t max_context; /* most tokens a sequence may hold: sizes what grows with a sequence (the pooled blocks of PS_MIX_WINATTN, a window of everything); 0: 65536 */
+    int32_t norm_groups; /* every RMS norm over the width is taken in this many equal consecutive parts, each with its own mean square (0 is taken as 1) */
 } ps_seq_desc;
 
 int ps_hip_seq_create(ps_hip_ctx *ctx, const ps_seq_desc *desc, ps_hip_seq **out);

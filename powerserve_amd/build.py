@@ -10,7 +10,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 OBJDIR = os.path.join(HERE, "build")
-SOURCES = ["ctx.hip", "api.hip", "model.hip", "k_quant.hip", "k_gemv.hip", "k_gemv4.hip", "k_qkvattn.hip", "k_gemvb.hip", "k_gemvk.hip", "k_gemm4k.hip", "k_gemv6.hip", "k_ops.hip", "k_attn.hip", "perf16.hip", "seqmodel.hip", "k_dense.hip", "k_seqmix.hip", "k_latent.hip", "k_winattn.hip"]
+SOURCES = ["ctx.hip", "api.hip", "model.hip", "k_quant.hip", "k_gemv.hip", "k_gemv4.hip", "k_qkvattn.hip", "k_gemvb.hip", "k_gemvk.hip", "k_gemm4k.hip", "k_gemv6.hip", "k_ops.hip", "k_attn.hip", "perf16.hip", "seqmodel.hip", "k_dense.hip", "k_seqmix.hip", "k_latent.hip", "k_winattn.hip", "k_moe.hip"]
 # -ffp-contract=off: the parity contract needs every fp32 op to round where the reference's C source rounds;
 # fused multiply-adds are written explicitly (__fmaf_rn) where the reference uses FMA intrinsics.
 # -fno-slp-vectorize (NOSLP files only): hipcc's SLP vectoriser packs adjacent scalar fp32 operations into v_pk_fma_f32 / v_pk_mul_f32 / v_pk_add_f32.  On
@@ -24,7 +24,7 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=o
          "-I" + os.path.join(HERE, "..", "include")]
 # The layer-list models (dense bf16 / fp32 matrices; include/ps_hip.h): their sources plus the context make a library of their own,
 # lib/libps_hip_seq.so, so that a checkout that only serves such a model compiles four files and not the quantized path's kernels.
-SEQ_SOURCES = ["ctx.hip", "seqmodel.hip", "k_dense.hip", "k_seqmix.hip", "k_latent.hip", "k_winattn.hip"]
+SEQ_SOURCES = ["ctx.hip", "seqmodel.hip", "k_dense.hip", "k_seqmix.hip", "k_latent.hip", "k_winattn.hip", "k_moe.hip"]
 # packed fp32 instructions are left to no one: these files are ordinary float code and are compiled without the feature
 SEQ_FLAGS = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 NOSLP = {"k_gemv4.hip", "k_qkvattn.hip", "k_gemvb.hip", "k_attn.hip", "k_gemm4k.hip"}  # k_gemm4k.hip (round 5): gate/up chunk launch of a 512-column sequence 384.2 -> 369-371 us, same bits (profiles/r05_g4k2_variants.txt, the "v2 0" lines vs profiles/r05_g4k_item_order.txt)  # (k_gemvb.hip: the Q4_0 / Q8_0 mat-vec, Llama-3.2-1B 1494 -> 1525 tok/s)

@@ -35,12 +35,23 @@ struct dn_args {
     float act_p, act_q, alpha;
     const float *mu, *shift0;
     int accum;
+    const float *out_scale;
+    // grouped products (ps_seq.h): N is one matrix's rows, wstride the elements between matrices
+    int groups, g_adiv, g_odiv, g_inner;
+    const int32_t *g_sel, *g_seg, *g_list;
+    const float *g_scale;
+    long long wstride;
 };
 
 // rows of A that exist and where they start (ring rows relative to the step's position)
 static __device__ __forceinline__ void dn_rows(const dn_args &g, long long &row0, int &T) {
     row0 = g.a_row0;
     T = g.T;
+    if (g.g_seg) { // the slots of matrix blockIdx.z: entries row0 .. row0 + T - 1 of the sorted list
+        row0 = g.g_seg[blockIdx.z];
+        T = g.g_seg[blockIdx.z + 1] - (int)row0;
+        return;
+    }
     if (g.a_step) {
         const long long p = g.a_step->pos0 + g.a_row0;
         row0 = p > 0 ? p : 0;
@@ -50,10 +61,12 @@ static __device__ __forceinline__ void dn_rows(const dn_args &g, long long &row0
 }
 static __device__ __forceinline__ const float *dn_arow(const dn_args &g, long long row0, int t) {
     long long r = row0 + t;
+    if (g.g_list) r = g.g_list[r] / g.g_adiv;
     if (g.a_mod > 0) r %= g.a_mod;
     return g.a + r * g.lda;
 }
 static __device__ __forceinline__ float dn_aval(const dn_args &g, long long row0, int t, long long k) {
+    if (g.g_list) return dn_arow(g, row0, t)[k] * (g.g_scale ? g.g_scale[g.g_list[row0 + t]] : 1.f);
     const float x = dn_arow(g, row0, t)[k];
     if (!g.mu) return x;
     const float p = t ? dn_arow(g, row0, t - 1)[k] : g.shift0[k];
@@ -72,19 +85,25 @@ static __device__ __forceinline__ float dn_epi(const dn_args &g, float acc, long
 static __device__ __forceinline__ float dn_silu(float x) { return x / (1.f + expf(-x)); }
 // Result acc of (token t, weight row n) goes to its place.  other: the result of row n ^ 1 (the paired activation needs both; every lane of the wave calls
 // this with both values, only the even row stores).
-static __device__ __forceinline__ void dn_put(const dn_args &g, int t, long long n, float acc, float other, bool in) {
+static __device__ __forceinline__ void dn_put(const dn_args &g, long long t, long long n, float acc, float other, bool in) {
+    const float rs = in && g.out_scale ? g.out_scale[t] : 1.f;
     if (g.act == PSD_ACT_SILU_PAIR) {
         if (in && !(n & 1)) {
-            float *p = g.out + (long long)t * g.ldo + (n >> 1);
-            const float v = dn_silu(acc) * other * g.alpha;
+            float *p = g.out + t * g.ldo + (n >> 1);
+            const float v = dn_silu(acc) * other * g.alpha * rs;
             *p = g.accum ? *p + v : v;
         }
         return;
     }
     if (!in) return;
-    float *p = g.out + (long long)t * g.ldo + n;
-    const float v = dn_epi(g, acc, n);
+    float *p = g.out + t * g.ldo + n;
+    const float v = dn_epi(g, acc, n) * rs;
     *p = g.accum ? *p + v : v;
+}
+// the output row of local row t (t < T): itself, or where the sorted list sends its slot
+static __device__ __forceinline__ long long dn_orow(const dn_args &g, long long row0, int t, int T) {
+    if (!g.g_list) return t;
+    return t < T ? g.g_list[row0 + t] / g.g_odiv : 0;
 }
 
 // ---------------------------------------------------------------------------------------------------- tiled mat-mul
@@ -106,7 +125,7 @@ __global__ __launch_bounds__(256) void dense_mm_kernel(dn_args g) {
     const long long n0 = (long long)blockIdx.x * 64;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
     const int lr = lane & 15, lq = lane >> 4;
-    const WT *W = (const WT *)g.w;
+    const WT *W = (const WT *)g.w + (g.g_seg ? (long long)blockIdx.z * g.wstride : 0);
     dn_f4 acc[2][2];
     for (int i = 0; i < 2; i++)
         for (int j = 0; j < 2; j++) acc[i][j] = dn_f4{0.f, 0.f, 0.f, 0.f};
@@ -179,7 +198,7 @@ __global__ __launch_bounds__(256) void dense_mm_kernel(dn_args g) {
             for (int e = 0; e < 4; e++) {
                 const int t = t0 + wm * 32 + i * 16 + lq * 4 + e;
                 const long long n = n0 + wn * 32 + j * 16 + lr;
-                dn_put(g, t, n, acc[i][j][e], __shfl_xor(acc[i][j][e], 1, 64), t < T && n < g.N); // (row n ^ 1 is the neighbouring lane's)
+                dn_put(g, dn_orow(g, row0, t, T), n, acc[i][j][e], __shfl_xor(acc[i][j][e], 1, 64), t < T && n < g.N); // (row n ^ 1 is the neighbouring lane's)
             }
 }
 
@@ -272,14 +291,85 @@ __global__ __launch_bounds__(256) void dense_mv_kernel(dn_args g) {
 }
 
 
+// Grouped mat-vec (ps_seq.h, grouped products): block row r = one output row, which adds its g_inner slots; slot s = r g_inner + i reads A row s / g_adiv
+// times g_scale[s] and the matrix g_sel[s].  Dynamic LDS: [g_inner][Kp] activations, rounded as in dense_mv_kernel.  The same four-rows-per-wave walk.
+template <typename WT>
+__global__ __launch_bounds__(256) void dense_mv_grouped_kernel(dn_args g) {
+    extern __shared__ __attribute__((aligned(16))) float xs[]; // [inner][Kp]
+    const long long K = g.K, Kp = (K + 7) / 8 * 8;
+    const int r = blockIdx.y, inner = g.g_inner;
+    for (long long i = threadIdx.x; i < (long long)inner * Kp; i += 256) {
+        const int c = (int)(i / Kp);
+        const long long k = i % Kp, s = (long long)r * inner + c;
+        float v = k < K ? g.a[(s / g.g_adiv) * g.lda + k] * (g.g_scale ? g.g_scale[s] : 1.f) : 0.f;
+        if constexpr (sizeof(WT) == 2) v = dn_bf2f(dn_f2bf(v));
+        xs[i] = v;
+    }
+    __syncthreads();
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    constexpr int RW = 4, VE = 16 / (int)sizeof(WT);
+    const bool vec = (K * (long long)sizeof(WT)) % 16 == 0;
+    for (long long nb = ((long long)blockIdx.x * 4 + wave) * RW; nb < g.N; nb += (long long)gridDim.x * 4 * RW) {
+        float acc[RW];
+#pragma unroll
+        for (int q = 0; q < RW; q++) acc[q] = 0.f;
+        for (int c = 0; c < inner; c++) {
+            const WT *W = (const WT *)g.w + (long long)g.g_sel[(long long)r * inner + c] * g.wstride;
+            const float *x = xs + (long long)c * Kp;
+            if (vec) {
+                for (long long k = (long long)lane * VE; k < K; k += 64 * VE) {
+                    dn_f4 raw[RW];
+#pragma unroll
+                    for (int q = 0; q < RW; q++) {
+                        const long long n = nb + q < g.N ? nb + q : g.N - 1;
+                        raw[q] = __builtin_nontemporal_load((const dn_f4 *)(W + n * K + k));
+                    }
+#pragma unroll
+                    for (int q = 0; q < RW; q++) {
+                        float wv[VE];
+                        if constexpr (sizeof(WT) == 2) {
+                            unsigned short h[8];
+                            __builtin_memcpy(h, &raw[q], 16);
+#pragma unroll
+                            for (int e = 0; e < 8; e++) wv[e] = dn_bf2f(h[e]);
+                        } else {
+                            __builtin_memcpy(wv, &raw[q], 16);
+                        }
+#pragma unroll
+                        for (int e = 0; e < VE; e++) acc[q] = fmaf(wv[e], x[k + e], acc[q]);
+                    }
+                }
+            } else {
+                for (long long k = lane; k < K; k += 64)
+#pragma unroll
+                    for (int q = 0; q < RW; q++) {
+                        const long long n = nb + q < g.N ? nb + q : g.N - 1;
+                        float wv;
+                        if constexpr (sizeof(WT) == 2) wv = dn_bf2f(((const unsigned short *)W)[n * K + k]);
+                        else wv = ((const float *)W)[n * K + k];
+                        acc[q] = fmaf(wv, x[k], acc[q]);
+                    }
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < RW; q++) {
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) acc[q] += __shfl_xor(acc[q], o, 64);
+        }
+#pragma unroll
+        for (int q = 0; q < RW; q++) dn_put(g, r, nb + q, acc[q], acc[q ^ 1], lane == 0 && nb + q < g.N);
+    }
+}
+
 // ---------------------------------------------------------------------------------------------------- wide mat-mul (bf16, K % 64 == 0)
 // The A operand is first packed to bfloat16 [Tp][K] (Tp = T rounded up to 128, rows beyond T zero; the ring rows and the token-shift mix
 // are resolved there), then 128 tokens x 128 outputs per work-group: four waves of 64 x 64 (4 x 4 tiles of v_mfma_f32_16x16x32_bf16), K in
 // steps of 64 through LDS (rows padded to 144 B), the next step's 16-byte global loads in flight while the matrix cores run the current one.
 __global__ __launch_bounds__(256) void dense_pack_kernel(dn_args g, unsigned short *out, int Tp) {
-    long long row0;
-    int T;
-    dn_rows(g, row0, T);
+    long long row0 = g.a_row0;
+    int T = g.T;
+    if (!g.g_list) dn_rows(g, row0, T); // (grouped: all T slots in the order of the sorted list, whatever their matrix)
+    else row0 = 0;
     const long long per_row = g.K / 8, total = (long long)Tp * per_row;
     for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long long)gridDim.x * 256) {
         const int t = (int)(i / per_row);
@@ -302,7 +392,8 @@ __global__ __launch_bounds__(256) void dense_mm_fast_kernel(dn_args g, const uns
     if (t0 >= T) return;
     const long long n0 = (long long)blockIdx.x * 128;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1, lr = lane & 15, lq = lane >> 4;
-    const unsigned short *W = (const unsigned short *)g.w;
+    const unsigned short *W = (const unsigned short *)g.w + (g.g_seg ? (long long)blockIdx.z * g.wstride : 0);
+    if (g.g_seg) A += row0 * g.K; // (the packed operand is in list order: this matrix's slots start at row0; a tile's rows beyond them are another matrix's or zero, and are not stored)
     const long long K = g.K;
     // staging: 128 rows x 64 k = 1024 pieces of 16 bytes per operand, four per thread: row = (tid >> 3) + 32 i, k piece = tid & 7
     const int sr = tid >> 3, sk = (tid & 7) * 8;
@@ -358,7 +449,7 @@ __global__ __launch_bounds__(256) void dense_mm_fast_kernel(dn_args g, const uns
             for (int e = 0; e < 4; e++) {
                 const int t = t0 + wm * 64 + i * 16 + lq * 4 + e;
                 const long long n = n0 + wn * 64 + j * 16 + lr;
-                dn_put(g, t, n, acc[i][j][e], __shfl_xor(acc[i][j][e], 1, 64), t < T && n < g.N);
+                dn_put(g, dn_orow(g, row0, t, T), n, acc[i][j][e], __shfl_xor(acc[i][j][e], 1, 64), t < T && n < g.N);
             }
 }
 
@@ -377,9 +468,41 @@ int psk_dense(hipStream_t st, const psk_dense_args &a) {
     dn_args g;
     g.w = a.w->data; g.a = a.a; g.lda = a.lda; g.a_row0 = a.a_row0; g.a_mod = a.a_mod; g.a_step = a.a_step; g.T = a.T;
     g.N = a.w->N; g.K = a.w->K; g.out = a.out; g.ldo = a.ldo; g.bias = a.bias; g.act = a.act; g.act_p = a.act_p; g.act_q = a.act_q;
-    g.alpha = a.alpha; g.mu = a.mu; g.shift0 = a.shift0; g.accum = a.accum;
+    g.alpha = a.alpha; g.mu = a.mu; g.shift0 = a.shift0; g.accum = a.accum; g.out_scale = a.out_scale;
+    g.groups = 0; g.g_adiv = 1; g.g_odiv = 1; g.g_inner = 1; g.g_sel = nullptr; g.g_seg = nullptr; g.g_list = nullptr; g.g_scale = nullptr; g.wstride = 0;
     const bool bf = a.w->dtype == PS_BF16;
     const size_t kp4 = (size_t)((g.K + 7) / 8 * 8) * 4;
+    if (a.groups > 0) {
+        g.groups = a.groups; g.N = a.w->N / a.groups; g.wstride = g.N * g.K;
+        g.g_adiv = a.g_adiv; g.g_odiv = a.g_odiv; g.g_inner = a.g_inner; g.g_sel = a.g_sel; g.g_scale = a.g_scale;
+        if (!a.g_list) { // a mat-vec per output row (T rows of g_inner slots each)
+            static unsigned long long mask = 0;
+            if (ps_first_on_device(&mask)) {
+                (void)hipFuncSetAttribute((const void *)dense_mv_grouped_kernel<unsigned short>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+                (void)hipFuncSetAttribute((const void *)dense_mv_grouped_kernel<float>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            }
+            long long blocks = (g.N + 15) / 16;
+            if (blocks > 2048) blocks = 2048;
+            const dim3 grid((unsigned)blocks, (unsigned)a.T);
+            if (bf) hipLaunchKernelGGL(dense_mv_grouped_kernel<unsigned short>, grid, dim3(256), kp4 * a.g_inner, st, g);
+            else hipLaunchKernelGGL(dense_mv_grouped_kernel<float>, grid, dim3(256), kp4 * a.g_inner, st, g);
+            return 0;
+        }
+        g.g_seg = a.g_seg; g.g_list = a.g_list;
+        const int Tp = (a.T + 127) / 128 * 128 + 128; // (a tile may start anywhere in the list and runs 127 rows on)
+        if (bf && !a.force_tiled && g.K % 64 == 0 && a.pack && (size_t)Tp * g.K * 2 <= a.pack_bytes) {
+            long long pb = ((long long)Tp * (g.K / 8) + 255) / 256;
+            if (pb > 8192) pb = 8192;
+            hipLaunchKernelGGL(dense_pack_kernel, dim3((unsigned)pb), dim3(256), 0, st, g, (unsigned short *)a.pack, Tp);
+            hipLaunchKernelGGL(dense_mm_fast_kernel, dim3((unsigned)((g.N + 127) / 128), (unsigned)((a.T + 127) / 128), (unsigned)a.groups), dim3(256), 0, st, g,
+                               (const unsigned short *)a.pack);
+            return 0;
+        }
+        const dim3 grid((unsigned)((g.N + 63) / 64), (unsigned)((a.T + 63) / 64), (unsigned)a.groups);
+        if (bf) hipLaunchKernelGGL(dense_mm_kernel<unsigned short>, grid, dim3(256), 0, st, g);
+        else hipLaunchKernelGGL(dense_mm_kernel<float>, grid, dim3(256), 0, st, g);
+        return 0;
+    }
     if (!a.force_tiled && a.T <= 8) {
         const int C = a.T <= 1 ? 1 : a.T <= 2 ? 2 : a.T <= 4 ? 4 : 8;
         if (kp4 * C <= 64 * 1024) {

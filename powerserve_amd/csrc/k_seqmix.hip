@@ -20,36 +20,88 @@ static __device__ __forceinline__ float sq_block_sum(float v, float *red) { // 2
 static __device__ __forceinline__ float sq_silu(float x) { return x / (1.f + expf(-x)); }
 static __device__ __forceinline__ float sq_softplus(float x) { return x > 20.f ? x : log1pf(expf(x)); }
 
+// (a row in `groups` equal consecutive parts, each with its own mean square: block (row, part) works on n = the part's length)
 __global__ __launch_bounds__(256) void sq_rmsnorm_kernel(const float *x, long long ldx, const int32_t *idx, const float *w, float offset, float eps, long long n,
                                                          float *y, long long ldy) {
     __shared__ float red[4];
-    const long long r = idx ? idx[blockIdx.x] : blockIdx.x;
-    const float *xr = x + r * ldx;
+    const long long r = idx ? idx[blockIdx.x] : blockIdx.x, part = (long long)blockIdx.y * n;
+    const float *xr = x + r * ldx + part;
+    w += part;
     float s = 0.f;
     for (long long i = threadIdx.x; i < n; i += 256) s += xr[i] * xr[i];
     s = sq_block_sum(s, red);
     const float inv = 1.f / sqrtf(s / (float)n + eps);
-    float *yr = y + (long long)blockIdx.x * ldy;
+    float *yr = y + (long long)blockIdx.x * ldy + part;
     for (long long i = threadIdx.x; i < n; i += 256) yr[i] = xr[i] * inv * (offset + w[i]);
 }
-void psk_rmsnorm(hipStream_t st, const float *x, int64_t ldx, const int32_t *idx, const float *w, float offset, float eps, int64_t n, int rows, float *y, int64_t ldy) {
+void psk_rmsnorm(hipStream_t st, const float *x, int64_t ldx, const int32_t *idx, const float *w, float offset, float eps, int64_t n, int rows, float *y, int64_t ldy,
+                 int groups) {
     if (rows <= 0) return;
-    hipLaunchKernelGGL(sq_rmsnorm_kernel, dim3(rows), dim3(256), 0, st, x, (long long)ldx, idx, w, offset, eps, (long long)n, y, (long long)ldy);
+    hipLaunchKernelGGL(sq_rmsnorm_kernel, dim3(rows, groups), dim3(256), 0, st, x, (long long)ldx, idx, w, offset, eps, (long long)(n / groups), y, (long long)ldy);
+}
+
+// The front of a parallel layer without an input filter, one block per row:  x = sum_j mix[j] X_j  over the nmix streams X_j = src + j stride (mix NULL: the last
+// of them as it is), kept in xout (NULL: not kept; it may be the last stream itself); then, over `groups` equal parts of the row each with its own mean square,
+// h = x / rms * (offset + w1) and h2 = x / rms * (offset + w2): two norms of the same vector share their statistics (w1 / w2 NULL: not wanted).
+// dynamic LDS: n + groups floats.
+__global__ __launch_bounds__(256) void sq_front_kernel(const float *src, long long stride, int nmix, const float *mix, const int32_t *idx, float *xout, const float *w1,
+                                                       float *h, const float *w2, float *h2, int groups, float offset, float eps, long long n) {
+    extern __shared__ float fr[];
+    float *xs = fr, *inv = fr + n;
+    const long long r = idx ? idx[blockIdx.x] : blockIdx.x, o = (long long)blockIdx.x * n;
+    const int tid = threadIdx.x;
+    for (long long i = tid; i < n; i += 256) {
+        float v;
+        if (mix) {
+            v = 0.f;
+            for (int j = 0; j < nmix; j++) v = fmaf(mix[j], src[j * stride + r * n + i], v);
+        } else {
+            v = src[(nmix - 1) * stride + r * n + i];
+        }
+        xs[i] = v;
+        if (xout) xout[o + i] = v;
+    }
+    if (!w1 && !w2) return;
+    __syncthreads();
+    const long long gs = n / groups;
+    for (int g = tid >> 6; g < groups; g += 4) {
+        float s = 0.f;
+        for (long long i = tid & 63; i < gs; i += 64) s += xs[g * gs + i] * xs[g * gs + i];
+#pragma unroll
+        for (int o2 = 32; o2 > 0; o2 >>= 1) s += __shfl_xor(s, o2, 64);
+        if ((tid & 63) == 0) inv[g] = 1.f / sqrtf(s / (float)gs + eps);
+    }
+    __syncthreads();
+    for (long long i = tid; i < n; i += 256) {
+        const float v = xs[i] * inv[i / gs];
+        if (w1) h[o + i] = v * (offset + w1[i]);
+        if (w2) h2[o + i] = v * (offset + w2[i]);
+    }
+}
+void psk_front(hipStream_t st, const float *src, int64_t stride, int nmix, const float *mix, const int32_t *idx, float *xout, const float *w1, float *h, const float *w2,
+               float *h2, int groups, float offset, float eps, int64_t n, int rows) {
+    if (rows <= 0) return;
+    static unsigned long long mask = 0;
+    if (ps_first_on_device(&mask)) (void)hipFuncSetAttribute((const void *)sq_front_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    hipLaunchKernelGGL(sq_front_kernel, dim3(rows), dim3(256), (size_t)(n + groups) * 4, st, src, (long long)stride, nmix, mix, idx, xout, w1, h, w2, h2, groups, offset, eps,
+                       (long long)n);
 }
 
 __global__ __launch_bounds__(256) void sq_norm_residual_kernel(float *x, const float *y, const float *w, float offset, float eps, long long n) {
     __shared__ float red[4];
-    const float *yr = y + (long long)blockIdx.x * n;
-    float *xr = x + (long long)blockIdx.x * n;
+    const long long at = ((long long)blockIdx.x * gridDim.y + blockIdx.y) * n; // (block (row, part) of a row of gridDim.y parts)
+    const float *yr = y + at;
+    float *xr = x + at;
+    w += (long long)blockIdx.y * n;
     float s = 0.f;
     for (long long i = threadIdx.x; i < n; i += 256) s += yr[i] * yr[i];
     s = sq_block_sum(s, red);
     const float inv = 1.f / sqrtf(s / (float)n + eps);
     for (long long i = threadIdx.x; i < n; i += 256) xr[i] += yr[i] * inv * (offset + w[i]);
 }
-void psk_norm_residual(hipStream_t st, float *x, const float *y, const float *w, float offset, float eps, int64_t n, int rows) {
+void psk_norm_residual(hipStream_t st, float *x, const float *y, const float *w, float offset, float eps, int64_t n, int rows, int groups) {
     if (rows <= 0) return;
-    hipLaunchKernelGGL(sq_norm_residual_kernel, dim3(rows), dim3(256), 0, st, x, y, w, offset, eps, (long long)n);
+    hipLaunchKernelGGL(sq_norm_residual_kernel, dim3(rows, groups), dim3(256), 0, st, x, y, w, offset, eps, (long long)(n / groups));
 }
 
 // ---------------------------------------------------------------------------------------------------- causal convolution with a tail
@@ -432,4 +484,51 @@ __global__ __launch_bounds__(64) void sq_headnorm_gate_kernel(float *o, long lon
 }
 void psk_headnorm_gate(hipStream_t st, float *o, int64_t ldo, const float *g, int64_t ldg, const float *w, int w_stride, float eps, int H, int dv, int T) {
     hipLaunchKernelGGL(sq_headnorm_gate_kernel, dim3(T, H), dim3(64), 0, st, o, (long long)ldo, g, (long long)ldg, w, w_stride, eps, dv);
+}
+
+
+// ---------------------------------------------------------------------------------------------------- element-wise gated recurrence (minGRU)
+// y[t] = [ z | u | g ] pre-activations (C each, row stride ldy).  Per channel  a_t = 1 - sigmoid(z_t),  b_t = sigmoid(z_t) cand(u_t)  with
+// cand(u) = u + 1/2 (u >= 0), sigmoid(u) (u < 0);  S_t = a_t S_(t-1) + b_t;  o[t] = S_t silu(g_t).  The state [C] is fp32 at step->state + state_off.
+// A block is 64 channels x NCH time chunks: every chunk first folds its own tokens from zero (A = prod a, B), the chunks' (A, B) meet in LDS, each chunk
+// takes the state in front of it and walks its tokens again, now storing.  One chunk (a short step): a single walk.
+static __device__ __forceinline__ float sq_sigmoid(float x) { return 1.f / (1.f + expf(-x)); }
+__global__ __launch_bounds__(1024) void sq_mingru_kernel(const ps_seq_step *step, long long state_off, const float *y, long long ldy, long long C, int T, float *o,
+                                                         long long ldo) {
+    __shared__ float As[16][64], Bs[16][64];
+    const int lane = threadIdx.x, ch = threadIdx.y, nch = blockDim.y;
+    const long long c = (long long)blockIdx.x * 64 + lane;
+    const bool in = c < C;
+    const int per = (T + nch - 1) / nch, tb = ch * per, te = min(T, tb + per);
+    const float *yz = y + c, *yu = y + C + c, *yg = y + 2 * C + c;
+    float *state = step->state + state_off;
+    float S = in ? state[c] : 0.f; // (read before the barrier below: the chunk with the last token overwrites it when it is done)
+    if (nch > 1) {
+        float A = 1.f, B = 0.f;
+        if (in)
+            for (int t = tb; t < te; t++) {
+                const float z = sq_sigmoid(yz[(long long)t * ldy]), u = yu[(long long)t * ldy];
+                const float cand = u >= 0.f ? u + 0.5f : sq_sigmoid(u), a = 1.f - z;
+                A *= a;
+                B = fmaf(a, B, z * cand);
+            }
+        As[ch][lane] = A;
+        Bs[ch][lane] = B;
+        __syncthreads();
+        if (in)
+            for (int j = 0; j < ch; j++) S = fmaf(As[j][lane], S, Bs[j][lane]);
+    }
+    if (!in) return;
+    for (int t = tb; t < te; t++) {
+        const float z = sq_sigmoid(yz[(long long)t * ldy]), u = yu[(long long)t * ldy], gg = yg[(long long)t * ldy];
+        const float cand = u >= 0.f ? u + 0.5f : sq_sigmoid(u);
+        S = fmaf(1.f - z, S, z * cand);
+        o[(long long)t * ldo + c] = S * sq_silu(gg);
+    }
+    if (te == T && tb < T) state[c] = S; // (the chunk that holds the last token)
+}
+void psk_mingru_scan(hipStream_t st, const ps_seq_step *step, int64_t state_off, const float *y, int64_t ldy, int64_t C, int T, float *o, int64_t ldo) {
+    const int nch = T >= 256 ? 16 : T >= 64 ? 8 : T >= 16 ? 4 : 1;
+    hipLaunchKernelGGL(sq_mingru_kernel, dim3((unsigned)((C + 63) / 64)), dim3(64, nch), 0, st, step, (long long)state_off, y, (long long)ldy, (long long)C, T, o,
+                       (long long)ldo);
 }

@@ -36,7 +36,7 @@ static __device__ __forceinline__ long long wa_blocks(long long p, int window, i
 // winattn_pool_kernel makes for a portion).  dynamic LDS: rot_dims floats (cos | sin of the token's angles, shared by all heads).
 __global__ __launch_bounds__(256) void winattn_prep_kernel(const ps_seq_step *step, long long ring_off, int cap, long long pool_off, int pool, const float *y,
                                                            long long ldy, const float *qnorm, const float *knorm, float eps, int H, int G, int d, int dv, int rot_dims,
-                                                           int pairing, const float *freq, float *qo, long long ldq) {
+                                                           int pairing, const float *freq, float *qo, long long ldq, float qt_coef, int qt_every) {
     extern __shared__ float cs[];
     __shared__ float red[8];
     const int t = blockIdx.x, tid = threadIdx.x;
@@ -44,6 +44,8 @@ __global__ __launch_bounds__(256) void winattn_prep_kernel(const ps_seq_step *st
     const int nq = H * d, nk = G * d, nv = G * dv, half = rot_dims / 2;
     const float *qt = y + (long long)t * ldy, *kt = qt + nq, *vt = kt + nk;
     float *ring = step->state + ring_off + (pos % cap) * (long long)(nk + nv);
+    // a query temperature that grows with the position in steps of qt_every tokens: 1 + coef ln(floor((pos + 1) / every) + 1)
+    const float qtemp = qt_every > 0 ? 1.f + qt_coef * logf((float)((pos + 1) / qt_every) + 1.f) : 1.f;
     for (int i = tid; i < half; i += 256) {
         const float ang = (float)pos * freq[i];
         cs[i] = cosf(ang);
@@ -82,7 +84,7 @@ __global__ __launch_bounds__(256) void winattn_prep_kernel(const ps_seq_step *st
     // the elements of q | k | v are spread over the blocks of a token (gridDim.y; every block has made the sums above for itself)
     for (int e = blockIdx.y * 256 + tid; e < nq + nk + nv; e += 256 * gridDim.y) {
         if (e < nq) {
-            qo[(long long)t * ldq + e] = turned(qt, qnorm, ia, e);
+            qo[(long long)t * ldq + e] = turned(qt, qnorm, ia, e) * qtemp;
         } else {
             const int i = e - nq;
             const float v = i < nk ? turned(kt, knorm, ib, i) : vt[i - nk];
@@ -108,11 +110,12 @@ __global__ __launch_bounds__(256) void winattn_pool_kernel(const ps_seq_step *st
 }
 
 void psk_winattn_prep(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int cap, int64_t pool_off, int pool, const float *y, int64_t ldy, const float *qnorm,
-                      const float *knorm, float eps, int H, int G, int d, int dv, int rot_dims, int pairing, const float *freq, int T, float *q, int64_t ldq) {
+                      const float *knorm, float eps, int H, int G, int d, int dv, int rot_dims, int pairing, const float *freq, int T, float *q, int64_t ldq, float qt_coef,
+                      int qt_every) {
     const int total = H * d + G * (d + dv);
     const int split = T >= 64 ? 1 : std::min(16, (total + 511) / 512); // few tokens: a token's elements over several blocks
     hipLaunchKernelGGL(winattn_prep_kernel, dim3(T, split), dim3(256), (size_t)(rot_dims + 2) * 4, st, step, (long long)ring_off, cap, (long long)pool_off, pool, y, (long long)ldy,
-                       qnorm, knorm, eps, H, G, d, dv, rot_dims, pairing, freq, q, (long long)ldq);
+                       qnorm, knorm, eps, H, G, d, dv, rot_dims, pairing, freq, q, (long long)ldq, qt_coef, qt_every);
     if (pool > 0 && T > 1) {
         const int rs = G * (d + dv);
         hipLaunchKernelGGL(winattn_pool_kernel, dim3((rs + 255) / 256, (T - 1) / pool + 2), dim3(256), 0, st, step, (long long)ring_off, cap, (long long)pool_off, pool, rs);
@@ -131,7 +134,7 @@ static __device__ __forceinline__ float wa_sigmoid(float x) { return 1.f / (1.f 
 #define WA_NV 4 // value columns per lane: dv <= 256
 __global__ __launch_bounds__(64) void winattn_kernel(const ps_seq_step *step, long long ring_off, int cap, long long pool_off, int pool, const float *q, long long ldq,
                                                      const float *gate, long long ldg, const float *temp, const float *sink, int H, int G, int d, int dv, int window,
-                                                     float scale, float *o, long long ldo) {
+                                                     float scale, float *o, long long ldo, float softcap) {
     extern __shared__ float lds[];
     float *qs = lds, *ps = lds + d;
     const int t = blockIdx.x, h = blockIdx.y, g = h / (H / G), lane = threadIdx.x;
@@ -154,6 +157,7 @@ __global__ __launch_bounds__(64) void winattn_kernel(const ps_seq_step *step, lo
             float a = 0.f;
             for (int i = 0; i < d; i++) a = fmaf(qs[i], kn[i], a);
             s = a * sc;
+            if (softcap > 0.f) s = softcap * tanhf(s / softcap);
         }
         const float mn = fmaxf(m, wa_wave_max(s));
         const float corr = expf(m - mn), pj = n < nkeys ? expf(s - mn) : 0.f;
@@ -179,9 +183,9 @@ __global__ __launch_bounds__(64) void winattn_kernel(const ps_seq_step *step, lo
         if (lane + 64 * x < dv) o[(long long)t * ldo + (long long)h * dv + lane + 64 * x] = acc[x] * f;
 }
 void psk_winattn(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int cap, int64_t pool_off, int pool, const float *q, int64_t ldq, const float *gate,
-                 int64_t ldg, const float *temp, const float *sink, int H, int G, int d, int dv, int window, float scale, int T, float *o, int64_t ldo) {
+                 int64_t ldg, const float *temp, const float *sink, int H, int G, int d, int dv, int window, float scale, int T, float *o, int64_t ldo, float softcap) {
     hipLaunchKernelGGL(winattn_kernel, dim3(T, H), dim3(64), (size_t)(d + 64) * 4, st, step, (long long)ring_off, cap, (long long)pool_off, pool, q, (long long)ldq, gate,
-                       (long long)ldg, temp, sink, H, G, d, dv, window, scale, o, (long long)ldo);
+                       (long long)ldg, temp, sink, H, G, d, dv, window, scale, o, (long long)ldo, softcap);
 }
 
 // ---------------------------------------------------------------------------------------------------- matrix-core forms (ps_attn_dev.h)
@@ -190,7 +194,7 @@ void psk_winattn(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int 
 template <int NJ>
 __global__ __launch_bounds__(256) void winattn_mfma_kernel(const ps_seq_step *step, long long ring_off, int cap, long long pool_off, int pool, const float *q, long long ldq,
                                                            const float *gate, long long ldg, const float *temp, const float *sink, int H, int G, int d, int dv, int window,
-                                                           float scale, int T, float *o, long long ldo) {
+                                                           float scale, int T, float *o, long long ldo, float softcap) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 15, lq = lane >> 4, h = blockIdx.y, g = h / (H / G);
     const int qld = d + 4;
@@ -226,12 +230,12 @@ __global__ __launch_bounds__(256) void winattn_mfma_kernel(const ps_seq_step *st
     const long long nbmax = wa_blocks(plast, window, pool);
     {
         const la_src k1 = {means + (long long)g * d, rs, 0, 0}, vs = {means + (long long)G * d + (long long)g * dv, rs, 0, 0};
-        for (long long j0 = 0; j0 < nbmax; j0 += 16) la_tile<NJ>(qs, qld, pt, k1, k1, vs, d, 0, dv, j0, nbmax, blo, bhi, sc, m, l, acc);
+        for (long long j0 = 0; j0 < nbmax; j0 += 16) la_tile<NJ>(qs, qld, pt, k1, k1, vs, d, 0, dv, j0, nbmax, blo, bhi, sc, m, l, acc, softcap);
     }
     {
         const la_src k1 = {ring + (long long)g * d, rs, 0, cap}, vs = {ring + (long long)G * d + (long long)g * dv, rs, 0, cap};
         const long long lo = pfirst - window + 1 > 0 ? pfirst - window + 1 : 0;
-        for (long long j0 = lo; j0 <= plast; j0 += 16) la_tile<NJ>(qs, qld, pt, k1, k1, vs, d, 0, dv, j0, plast + 1, rowlo, rowhi, sc, m, l, acc);
+        for (long long j0 = lo; j0 <= plast; j0 += 16) la_tile<NJ>(qs, qld, pt, k1, k1, vs, d, 0, dv, j0, plast + 1, rowlo, rowhi, sc, m, l, acc, softcap);
     }
 #pragma unroll
     for (int i = 0; i < 4; i++) {
@@ -250,11 +254,11 @@ static size_t wa_mfma_lds(int d) { return (size_t)4 * (16 * (d + 4) + 16 * 17) *
 // the sizes the matrix-core forms take: 16-byte pieces of keys (d a multiple of 16) and values (dv of 4, at most 128 columns per head)
 bool psk_winattn_mfma_ok(int d, int dv) { return d % 16 == 0 && dv % 4 == 0 && dv <= 128 && wa_mfma_lds(d) <= 160 * 1024; }
 void psk_winattn_mfma(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int cap, int64_t pool_off, int pool, const float *q, int64_t ldq, const float *gate,
-                      int64_t ldg, const float *temp, const float *sink, int H, int G, int d, int dv, int window, float scale, int T, float *o, int64_t ldo) {
+                      int64_t ldg, const float *temp, const float *sink, int H, int G, int d, int dv, int window, float scale, int T, float *o, int64_t ldo, float softcap) {
     static unsigned long long mask = 0;
     if (ps_first_on_device(&mask)) (void)hipFuncSetAttribute((const void *)winattn_mfma_kernel<8>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     hipLaunchKernelGGL(winattn_mfma_kernel<8>, dim3((T + 63) / 64, H), dim3(256), wa_mfma_lds(d), st, step, (long long)ring_off, cap, (long long)pool_off, pool, q,
-                       (long long)ldq, gate, (long long)ldg, temp, sink, H, G, d, dv, window, scale, T, o, (long long)ldo);
+                       (long long)ldq, gate, (long long)ldg, temp, sink, H, G, d, dv, window, scale, T, o, (long long)ldo, softcap);
 }
 
 // A single token.  Rows = the heads that share key / value group g (16 per block); the keys are cut into tiles of 16 in one index space -- tiles
@@ -263,7 +267,7 @@ void psk_winattn_mfma(hipStream_t st, const ps_seq_step *step, int64_t ring_off,
 // dynamic LDS: 16 x (d + 4) + 4 x 16 x 17
 template <int NJ>
 __global__ __launch_bounds__(256) void winattn_step_kernel(const ps_seq_step *step, long long ring_off, int cap, long long pool_off, int pool, const float *q,
-                                                           const float *temp, int H, int G, int d, int dv, int window, float scale, float *part) {
+                                                           const float *temp, int H, int G, int d, int dv, int window, float scale, float *part, float softcap) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 15, lq = lane >> 4, g = blockIdx.z, hpg = H / G, r0 = blockIdx.y * 16;
     const int qld = d + 4;
@@ -289,7 +293,7 @@ __global__ __launch_bounds__(256) void winattn_step_kernel(const ps_seq_step *st
     for (int i = 0; i < 4; i++) { const bool in = r0 + 4 * lq + i < hpg; rowlo[i] = 0; rowhi[i] = in ? jend : 0; m[i] = -INFINITY; l[i] = 0.f; }
 #pragma unroll
     for (int j = 0; j < NJ; j++) acc[j] = la_f4{0.f, 0.f, 0.f, 0.f};
-    la_tile<NJ>(qs, qld, pt, k1, k1, vs, d, 0, dv, j0, jend, rowlo, rowhi, scale, m, l, acc);
+    la_tile<NJ>(qs, qld, pt, k1, k1, vs, d, 0, dv, j0, jend, rowlo, rowhi, scale, m, l, acc, softcap);
     const int dvp = dv + 4;
 #pragma unroll
     for (int i = 0; i < 4; i++) {
@@ -349,12 +353,12 @@ size_t psk_winattn_step_scratch(int H, int dv, int window, int pool, int64_t max
 }
 // q [H * d] -> o [H * dv]; gate [H] raw or NULL; scratch from psk_winattn_step_scratch
 void psk_winattn_step(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int cap, int64_t pool_off, int pool, const float *q, const float *gate, const float *temp,
-                      const float *sink, int H, int G, int d, int dv, int window, float scale, int64_t max_context, float *scratch, float *o) {
+                      const float *sink, int H, int G, int d, int dv, int window, float scale, int64_t max_context, float *scratch, float *o, float softcap) {
     const int max_tiles = wa_max_tiles(window, pool, max_context);
     const size_t lds = (size_t)(16 * (d + 4) + 4 * 16 * 17) * 4;
     static unsigned long long mask = 0;
     if (ps_first_on_device(&mask)) (void)hipFuncSetAttribute((const void *)winattn_step_kernel<8>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     const dim3 grid((max_tiles + 3) / 4, (H / G + 15) / 16, G);
-    hipLaunchKernelGGL(winattn_step_kernel<8>, grid, dim3(256), lds, st, step, (long long)ring_off, cap, (long long)pool_off, pool, q, temp, H, G, d, dv, window, scale, scratch);
+    hipLaunchKernelGGL(winattn_step_kernel<8>, grid, dim3(256), lds, st, step, (long long)ring_off, cap, (long long)pool_off, pool, q, temp, H, G, d, dv, window, scale, scratch, softcap);
     hipLaunchKernelGGL(winattn_merge_kernel, dim3(H), dim3(256), (size_t)grid.x * 4 * 4, st, step, scratch, gate, sink, pool, H, dv, window, (int)grid.x * 4, o);
 }

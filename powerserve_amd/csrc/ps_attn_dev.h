@@ -29,7 +29,7 @@ static __device__ __forceinline__ const float *la_row(const la_src &s, long long
 template <int NJ>
 static __device__ __forceinline__ void la_tile(const float *qs, int qld, float *pt, const la_src &k1, const la_src &k2, const la_src &vs, int DK1, int DK2, int DV,
                                                long long j0, long long jend, const long long (&rowlo)[4], const long long (&rowhi)[4], float scale, float (&m)[4], float (&l)[4],
-                                               la_f4 (&acc)[NJ]) {
+                                               la_f4 (&acc)[NJ], float softcap = 0.f) { // softcap > 0: score <- softcap tanh(score / softcap) behind the scale
     const int lane = threadIdx.x & 63, lr = lane & 15, lq = lane >> 4;
     const long long jk = j0 + lr < jend ? j0 + lr : jend - 1; // (a key row that exists; masked below)
     la_f4 s4 = {0.f, 0.f, 0.f, 0.f};
@@ -59,7 +59,9 @@ static __device__ __forceinline__ void la_tile(const float *qs, int qld, float *
 #pragma unroll
     for (int i = 0; i < 4; i++) {
         const bool vis = j < jend && j >= rowlo[i] && j < rowhi[i];
-        const float s = vis ? s4[i] * scale : -INFINITY;
+        float sv = s4[i] * scale;
+        if (softcap > 0.f) sv = softcap * tanhf(sv / softcap);
+        const float s = vis ? sv : -INFINITY;
         float tm = s;
 #pragma unroll
         for (int o = 1; o < 16; o <<= 1) tm = fmaxf(tm, __shfl_xor(tm, o, 64));

@@ -44,6 +44,15 @@ struct psk_dense_args {
     int force_tiled = 0; // 1: the plain tiled mat-mul whatever the shape (A/B against the mat-vec and the wide mat-mul)
     void *pack = nullptr; // scratch for the wide mat-mul's bfloat16 copy of A (T rounded up to 128 rows of K); without it the plain tiled kernel runs
     size_t pack_bytes = 0;
+    const float *out_scale = nullptr; // [T] device: row t of the result is multiplied by out_scale[t] (beside alpha)
+    // ---- grouped products: w holds `groups` matrices of N / groups rows one after the other, and every row of the product belongs to one of them.
+    // T counts SLOTS; slot s reads A row s / g_adiv times g_scale[s] (NULL: 1), uses matrix g_sel[s] and lands in output row s / g_odiv.
+    // More than 8 slots: the slots sorted by matrix come as g_list with g_seg [groups + 1] (moe plan), a tile never mixes matrices; g_odiv > 1 is then not
+    // taken (two slots of a row would meet: the caller sums per-slot results).  At most 8 slots x g_inner: a mat-vec per output row, which adds the g_inner
+    // slots r g_inner .. r g_inner + g_inner - 1 of row r (T counts rows there, g_odiv is ignored).
+    int groups = 0, g_adiv = 1, g_odiv = 1, g_inner = 1;
+    const int32_t *g_sel = nullptr, *g_seg = nullptr, *g_list = nullptr;
+    const float *g_scale = nullptr;
 };
 int psk_dense(hipStream_t st, const psk_dense_args &a);
 void psk_dense_widen(hipStream_t st, const uint16_t *bf16, int64_t n, float *out);
@@ -54,9 +63,19 @@ void psk_argmax_rows(hipStream_t st, const float *x, int64_t n, int rows, int32_
 
 // ---- k_seqmix.hip
 // y[r] = x[row(r)] / sqrt(mean(x^2) + eps) * (offset + w),  row(r) = idx ? idx[r] : r
-void psk_rmsnorm(hipStream_t st, const float *x, int64_t ldx, const int32_t *idx, const float *w, float offset, float eps, int64_t n, int rows, float *y, int64_t ldy);
+//   (groups > 1: the row in that many equal consecutive parts, each divided by its own root mean square)
+void psk_rmsnorm(hipStream_t st, const float *x, int64_t ldx, const int32_t *idx, const float *w, float offset, float eps, int64_t n, int rows, float *y, int64_t ldy,
+                 int groups = 1);
 // x[r] += y[r] / sqrt(mean(y^2) + eps) * (offset + w)
-void psk_norm_residual(hipStream_t st, float *x, const float *y, const float *w, float offset, float eps, int64_t n, int rows);
+void psk_norm_residual(hipStream_t st, float *x, const float *y, const float *w, float offset, float eps, int64_t n, int rows, int groups = 1);
+// The front of a parallel layer that has no input filter, in one launch: x[r] = sum_j mix[j] X_j[row(r)] over the nmix streams X_j = src + j stride (mix NULL:
+// the last stream alone), row(r) = idx ? idx[r] : r, stored to xout[r] (NULL: not kept); then h[r] = norm(x) (offset + w1) and h2[r] = norm(x) (offset + w2) with
+// the norm taken over `groups` parts -- two norms of one vector share their statistics.  w1 / w2 NULL: that output is not made.
+void psk_front(hipStream_t st, const float *src, int64_t stride, int nmix, const float *mix, const int32_t *idx, float *xout, const float *w1, float *h, const float *w2,
+               float *h2, int groups, float offset, float eps, int64_t n, int rows);
+// Element-wise gated recurrence.  y[t] = [ z | u | g ] (C each): S <- (1 - sigmoid(z)) S + sigmoid(z) c(u), c(u) = sigmoid(u) for negative u, else u + 0.5;
+// o[t] = S silu(g).  State [C] fp32 at step->state + state_off.
+void psk_mingru_scan(hipStream_t st, const ps_seq_step *step, int64_t state_off, const float *y, int64_t ldy, int64_t C, int T, float *o, int64_t ldo);
 // Causal convolution over time on each channel, taps taken from the step's rows and, before them, from the sequence's tail (the last taps - 1
 // inputs of earlier steps, [taps - 1][C] at step->state + tail_off): out[t][c] = f(sum_j w[c][j] in(t - taps + 1 + j)[c]); mode 0: f = in(t) + sum
 // (a residual around the convolution), mode 1: f = silu(sum).  The tail is brought up to date behind it.
@@ -86,6 +105,16 @@ void psk_delta_scan(hipStream_t st, const ps_seq_step *step, int64_t state_off, 
 // o[t][h][:] = o / sqrt(mean_j o^2 + eps) * w(h, :) * silu(g[t][h][:]);  w_stride = dv (a weight per head) or 0 (one shared by the heads)
 void psk_headnorm_gate(hipStream_t st, float *o, int64_t ldo, const float *g, int64_t ldg, const float *w, int w_stride, float eps, int H, int dv, int T);
 
+// ---- k_moe.hip
+// Router of a mixture of experts, fp32: scores = sigmoid(router h[t]); the `top` largest (ties: the lower index) -> sel[t top + i], wgt[t top + i] (their scores,
+// divided by their sum where norm_top); sgate[t] = sigmoid(shared_gate . h[t]) where shared_gate is given.
+void psk_moe_route(hipStream_t st, const float *h, int64_t ldh, const float *router, const float *shared_gate, int experts, int top, int norm_top, int64_t K, int T,
+                   int32_t *sel, float *wgt, float *sgate);
+// The S slots sorted by expert: seg [experts + 1] (slots of expert e are list[seg[e] .. seg[e + 1])), list [S]
+void psk_moe_plan(hipStream_t st, const int32_t *sel, int S, int experts, int32_t *seg, int32_t *list);
+// x[t] += alpha * sum_i y[t top + i]
+void psk_moe_combine(hipStream_t st, float *x, const float *y, int top, float alpha, int64_t n, int T);
+
 // ---- k_latent.hip
 // One token per block.  y[t] = [ dq (q_rank) | ckv (kv_rank) | kr (rot_dim) ]:  cq[t] = rmsnorm(dq) * qnorm;  ring row (pos mod cap):
 // c = rmsnorm(ckv) * kvnorm, kr with its first rot_dims numbers rotated at pos (pairs (i, i + rot_dims/2), angle pos * freq[i]).  Ring at step->state + ring_off: [cap][kv_rank + rot_dim].
@@ -111,16 +140,19 @@ void psk_latent_absorbed(hipStream_t st, const ps_seq_step *step, int64_t ring_o
 // every head at the token's position (pairing: ps_rot_pairing; angle of pair i: pos * freq[i]); q -> q[t], k and v -> the ring row pos mod cap ([G d | G dv], ring at
 // step->state + ring_off); then the block means ([block][G d | G dv] at step->state + pool_off, pool > 0) are brought up to date.
 void psk_winattn_prep(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int cap, int64_t pool_off, int pool, const float *y, int64_t ldy, const float *qnorm,
-                      const float *knorm, float eps, int H, int G, int d, int dv, int rot_dims, int pairing, const float *freq, int T, float *q, int64_t ldq);
+                      const float *knorm, float eps, int H, int G, int d, int dv, int rot_dims, int pairing, const float *freq, int T, float *q, int64_t ldq,
+                      float qt_coef = 0.f, int qt_every = 0); // qt_every > 0: q[t] times 1 + qt_coef ln(floor((pos + 1) / qt_every) + 1)
 // o[t][h] = gate(t, h) * soft-max attention of q[t][h] over the visible block means and the window's ring rows, scores times scale * temp[h], exp(sink[h]) in the
 // denominator; gate [T][..] raw (sigmoid here; column h, row stride ldg), temp / sink / gate may be NULL.
 void psk_winattn(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int cap, int64_t pool_off, int pool, const float *q, int64_t ldq, const float *gate,
-                 int64_t ldg, const float *temp, const float *sink, int H, int G, int d, int dv, int window, float scale, int T, float *o, int64_t ldo);
+                 int64_t ldg, const float *temp, const float *sink, int H, int G, int d, int dv, int window, float scale, int T, float *o, int64_t ldo,
+                 float softcap = 0.f); // softcap > 0 (all three forms): score <- softcap tanh(score / softcap) behind scale and temperature
 // The same attention on the fp32 matrix cores for a portion, 16 tokens of a head per wave; _ok: the sizes it takes (d a multiple of 16, dv of 4, dv <= 128).
 bool psk_winattn_mfma_ok(int d, int dv);
 void psk_winattn_mfma(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int cap, int64_t pool_off, int pool, const float *q, int64_t ldq, const float *gate,
-                      int64_t ldg, const float *temp, const float *sink, int H, int G, int d, int dv, int window, float scale, int T, float *o, int64_t ldo);
+                      int64_t ldg, const float *temp, const float *sink, int H, int G, int d, int dv, int window, float scale, int T, float *o, int64_t ldo,
+                      float softcap = 0.f);
 // A single token on the matrix cores: rows = the heads of a key / value group, the keys spread over waves, partials merged in a second launch (same sizes).
 size_t psk_winattn_step_scratch(int H, int dv, int window, int pool, int64_t max_context);
 void psk_winattn_step(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int cap, int64_t pool_off, int pool, const float *q, const float *gate, const float *temp,
-                      const float *sink, int H, int G, int d, int dv, int window, float scale, int64_t max_context, float *scratch, float *o);
+                      const float *sink, int H, int G, int d, int dv, int window, float scale, int64_t max_context, float *scratch, float *o, float softcap = 0.f);

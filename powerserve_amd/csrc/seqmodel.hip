@@ -5,9 +5,13 @@
 // or PARALLEL,  h = norm(x); x += mixer(conv(h)) + ff(h).  A layer's mixer may have a second one beside it that reads the same input
 // (their outputs are added, each times its scale), and a stretch of layers may run several times in a row with the same weights: the
 // unit that owns state is the layer RUN.  What a sequence carries: per run the tails of the input convolutions, and per mixer kind a
-// token-shift row + the wkv state, the short convolutions' tail + the delta-rule state, the gated-linear-attention state, the ring of
-// latents, or the ring of keys and values + the block means -- one fp32 block per slot, rings and means last, the rest zeroed when
-// the slot is handed out.
+// token-shift row + the wkv state, the short convolutions' tail + the delta-rule state, the gated-linear-attention state, the element-wise
+// recurrence's state, the ring of latents, or the ring of keys and values + the block means -- one fp32 block per slot, rings and means last,
+// the rest zeroed when the slot is handed out.
+// A parallel layer may go without the input filter, take its two sublayers' inputs from two norms of the same vector, scale the sublayers' sum, and
+// hand on a weighted average of ALL earlier layers' results instead of its own (depth_mix): the results X_0 .. X_runs of a portion then live side by
+// side (`hist`), a layer's sublayers add into its own X, and the average, the next layer's norms and their group statistics are one launch (psk_front).
+// The feed-forward may be a mixture of experts: the router (fp32) picks per token, the experts' products are grouped launches of the dense kernels.
 #include "ps_seq.h"
 
 #include <cmath>
@@ -50,6 +54,10 @@ struct ps_hip_seq {
     float *x = nullptr, *hn = nullptr, *h = nullptr, *y = nullptr, *t1 = nullptr, *t2 = nullptr, *t3 = nullptr, *t4 = nullptr, *kvx = nullptr, *xn = nullptr,
           *logits = nullptr;
     int32_t *tokens = nullptr, *want = nullptr, *amax = nullptr, *ids = nullptr;
+    float *hist = nullptr;        // depth_mix: [runs + 1][max_batch][width], X_0 = the embedding, run i writes X_(i+1)
+    int groups = 1;               // parts of every RMS norm over the width
+    int32_t *moe_sel = nullptr, *moe_seg = nullptr, *moe_list = nullptr; // mixture of experts: expert per slot, the slots sorted by expert
+    float *moe_wgt = nullptr, *moe_sg = nullptr, *moe_y = nullptr;       // weight per slot, the shared expert's gate per token, per-slot results (top > 1)
     float *win_scratch = nullptr; // the windowed attention's single-token partials
     float *abs_scratch = nullptr; // the absorbed single-token attention's folded queries, attended latents and per-tile partials
     void *pack = nullptr; // the wide mat-mul's bfloat16 operand copy
@@ -98,6 +106,10 @@ int ps_hip_seq_create(ps_hip_ctx *c, const ps_seq_desc *desc, ps_hip_seq **out) 
     auto shape = [](const ps_dense *w, int64_t N, int64_t K) { return w && w->N == N && w->K == K; };
     m->max_context = desc->max_context > 0 ? desc->max_context : 65536;
     m->embed_scale = desc->embed_scale != 0.f ? desc->embed_scale : 1.f;
+    m->groups = desc->norm_groups > 0 ? desc->norm_groups : 1;
+    if (W % m->groups) return fail("norm_groups does not divide the width");
+    int64_t moe_slots = 0, moe_experts = 0, moe_top = 1;
+    bool depth = false;
     std::vector<int> order; // layer index of every run
     {
         const bool loop = desc->loop_times > 1;
@@ -183,6 +195,13 @@ int ps_hip_seq_create(ps_hip_ctx *c, const ps_seq_desc *desc, ps_hip_seq **out) 
             n2 = std::max(n2, H * d);
             n3 = std::max(n3, H * dv);
             m->weight_bytes += dense_bytes(l.in_cat) + dense_bytes(l.decay2) + dense_bytes(l.out);
+        } else if (l.kind == PS_MIX_MINGRU) {
+            P.ncat = 3 * d;
+            if (!shape(l.in_cat, P.ncat, W) || !shape(l.out, W, d)) return at + "gated recurrence tensors";
+            P.off_S = off; off += d;
+            n1 = std::max(n1, P.ncat);
+            n3 = std::max(n3, d);
+            m->weight_bytes += dense_bytes(l.in_cat) + dense_bytes(l.out);
         } else {
             return at + "unknown mixer kind";
         }
@@ -196,12 +215,32 @@ int ps_hip_seq_create(ps_hip_ctx *c, const ps_seq_desc *desc, ps_hip_seq **out) 
         const ps_seq_layer &l = P.d;
         const std::string at = "layer " + std::to_string(P.layer) + ": ";
         if (l.form != PS_LAYER_SEQUENTIAL && l.form != PS_LAYER_PARALLEL) return fail(at + "unknown layer form");
-        if (!l.norm1 || (l.form == PS_LAYER_SEQUENTIAL && !l.norm1b) || !l.canon1) return fail(at + "norm / canon missing");
-        P.off_canon1 = off; off += (int64_t)(desc->canon_taps - 1) * W;
+        if (!l.norm1 || (l.form == PS_LAYER_SEQUENTIAL && !l.norm1b) || (l.form == PS_LAYER_SEQUENTIAL && !l.canon1)) return fail(at + "norm / canon missing");
+        if (l.canon1) { P.off_canon1 = off; off += (int64_t)(desc->canon_taps - 1) * W; }
+        if (l.canon1 && (l.norm2 && l.form == PS_LAYER_PARALLEL)) return fail(at + "a parallel layer with an input filter has one norm");
+        if (l.depth_mix) {
+            if (l.form != PS_LAYER_PARALLEL || l.canon1 || desc->loop_times > 1) return fail(at + "depth_mix needs parallel layers without an input filter and no loop");
+            depth = true;
+        }
         if (l.ff_kind != PS_FF_NONE) {
-            if (l.ff_kind != PS_FF_DENSE_XIELU && l.ff_kind != PS_FF_DENSE_SWIGLU) return fail(at + "unknown feed-forward kind");
+            if (l.ff_kind != PS_FF_DENSE_XIELU && l.ff_kind != PS_FF_DENSE_SWIGLU && l.ff_kind != PS_FF_MOE_SWIGLU) return fail(at + "unknown feed-forward kind");
+            const bool moe = l.ff_kind == PS_FF_MOE_SWIGLU;
+            if (moe) {
+                if (l.form != PS_LAYER_PARALLEL || l.canon1) return fail(at + "a mixture of experts needs a parallel layer without an input filter");
+                if (l.experts <= 0 || l.top <= 0 || l.top > l.experts || l.ff <= 0 || !l.router) return fail(at + "mixture-of-experts sizes / router");
+                if (!shape(l.ff_up, (int64_t)l.experts * 2 * l.ff, W) || !shape(l.ff_down, (int64_t)l.experts * W, l.ff)) return fail(at + "expert tensors");
+                if (l.shared_up || l.shared_down) {
+                    if (l.shared_ff <= 0 || !shape(l.shared_up, 2 * (int64_t)l.shared_ff, W) || !shape(l.shared_down, W, l.shared_ff)) return fail(at + "shared expert tensors");
+                    m->weight_bytes += dense_bytes(l.shared_up) + dense_bytes(l.shared_down);
+                }
+                moe_slots = std::max(moe_slots, B * l.top);
+                moe_experts = std::max<int64_t>(moe_experts, l.experts);
+                moe_top = std::max<int64_t>(moe_top, l.top);
+                n4 = std::max<int64_t>({n4, (int64_t)l.top * l.ff, (int64_t)l.shared_ff});
+                m->weight_bytes += (dense_bytes(l.ff_up) + dense_bytes(l.ff_down)) / l.experts * l.top + (uint64_t)l.experts * W * 4;
+            }
             const int64_t up_rows = l.ff_kind == PS_FF_DENSE_SWIGLU ? 2 * (int64_t)l.ff : l.ff;
-            if (!shape(l.ff_up, up_rows, W) || !shape(l.ff_down, W, l.ff)) return fail(at + "feed-forward tensors");
+            if (!moe && (!shape(l.ff_up, up_rows, W) || !shape(l.ff_down, W, l.ff))) return fail(at + "feed-forward tensors");
             if (l.form == PS_LAYER_SEQUENTIAL) {
                 if (!l.norm2 || !l.norm2b || !l.canon2) return fail(at + "feed-forward norm / canon missing");
                 P.off_canon2 = off; off += (int64_t)(desc->canon_taps - 1) * W;
@@ -209,7 +248,7 @@ int ps_hip_seq_create(ps_hip_ctx *c, const ps_seq_desc *desc, ps_hip_seq **out) 
             const double sp = log1p(exp((double)l.ff_act_p)), sq = log1p(exp((double)l.ff_act_q));
             P.act_p = (float)sp; P.act_q = (float)(0.5 + sq);
             n4 = std::max<int64_t>(n4, l.ff);
-            m->weight_bytes += dense_bytes(l.ff_up) + dense_bytes(l.ff_down);
+            if (!moe) m->weight_bytes += dense_bytes(l.ff_up) + dense_bytes(l.ff_down);
         }
         std::string e = plan_mixer(P, at);
         if (!e.empty()) return fail(e);
@@ -223,6 +262,9 @@ int ps_hip_seq_create(ps_hip_ctx *c, const ps_seq_desc *desc, ps_hip_seq **out) 
         }
     }
     n2 = std::max(n2, m->n_t2q + nq);
+    if (depth)
+        for (auto &P : m->L)
+            if (P.d.form != PS_LAYER_PARALLEL || P.d.canon1) return fail("depth_mix needs every layer parallel and without an input filter");
     m->zero_floats = off;
     auto mixers = [&](auto &&f) { // every mixer plan, second ones included
         for (auto &P : m->L) { f(P); if (P.side) f(*P.side); }
@@ -258,7 +300,7 @@ int ps_hip_seq_create(ps_hip_ctx *c, const ps_seq_desc *desc, ps_hip_seq **out) 
     });
     {
         // the stacked input projections of two mixers side by side, joined once per layer (its runs share the copy)
-        auto stacked = [](int kind) { return kind == PS_MIX_WINATTN || kind == PS_MIX_GLA || kind == PS_MIX_DELTA; };
+        auto stacked = [](int kind) { return kind == PS_MIX_WINATTN || kind == PS_MIX_GLA || kind == PS_MIX_DELTA || kind == PS_MIX_MINGRU; };
         std::map<int, std::pair<const ps_dense *, const float *>> joint_of;
         for (auto &P : m->L) {
             if (!ok || !P.side || !stacked(P.d.kind) || !stacked(P.side->d.kind) || P.d.in_cat->dtype != P.side->d.in_cat->dtype) continue;
@@ -294,6 +336,10 @@ int ps_hip_seq_create(ps_hip_ctx *c, const ps_seq_desc *desc, ps_hip_seq **out) 
          alloc((void **)&m->t3, B * std::max<int64_t>(n3, 1) * 4) && alloc((void **)&m->t4, B * std::max<int64_t>(n4, 1) * 4) &&
          alloc((void **)&m->kvx, std::max<int64_t>(nkv, 1) * 4) && alloc((void **)&m->xn, B * W * 4) && alloc((void **)&m->logits, B * (int64_t)desc->vocab * 4) &&
          alloc((void **)&m->tokens, B * 4) && alloc((void **)&m->want, B * 4) && alloc((void **)&m->amax, B * 4);
+    if (depth) ok = ok && alloc((void **)&m->hist, (size_t)(order.size() + 1) * B * W * 4);
+    if (moe_slots)
+        ok = ok && alloc((void **)&m->moe_sel, moe_slots * 4) && alloc((void **)&m->moe_list, moe_slots * 4) && alloc((void **)&m->moe_seg, (moe_experts + 1) * 4) &&
+             alloc((void **)&m->moe_wgt, moe_slots * 4) && alloc((void **)&m->moe_sg, B * 4) && (moe_top <= 1 || alloc((void **)&m->moe_y, moe_slots * W * 4));
     {
         size_t ab = 0;
         mixers([&](LayerPlan &P) {
@@ -311,10 +357,11 @@ int ps_hip_seq_create(ps_hip_ctx *c, const ps_seq_desc *desc, ps_hip_seq **out) 
     if (desc->compute == 0) { // the wide mat-mul's operand copy: the widest input of any matrix x a portion's rows, or the window's rows x the latent
         int64_t kmax = W, kvrows = 0, kvk = 0;
         mixers([&](LayerPlan &P) {
-            kmax = std::max<int64_t>({kmax, P.d.ff, P.d.heads * (int64_t)std::max(P.d.dim, P.d.vdim), P.d.q_rank, P.d.decay_rank});
+            kmax = std::max<int64_t>({kmax, P.d.ff, P.d.shared_ff, P.d.heads * (int64_t)std::max(P.d.dim, P.d.vdim), P.d.q_rank, P.d.decay_rank});
             if (P.d.kind == PS_MIX_LATENT) { kvrows = std::max<int64_t>(kvrows, P.d.window - 1 + B); kvk = std::max<int64_t>(kvk, P.d.kv_rank); }
         });
-        const int64_t r128 = (B + 127) / 128 * 128, kv128 = (kvrows + 127) / 128 * 128;
+        // (a grouped product packs its slots in list order and a tile may start anywhere in the list: one tile of rows more)
+        const int64_t r128 = std::max((B + 127) / 128 * 128, moe_slots ? (moe_slots + 127) / 128 * 128 + 128 : 0), kv128 = (kvrows + 127) / 128 * 128;
         m->pack_bytes = (size_t)std::max(r128 * kmax, kv128 * kvk) * 2;
         ok = ok && alloc(&m->pack, m->pack_bytes);
     }
@@ -372,7 +419,8 @@ static void seq_layers(ps_hip_seq *m, float *state, int T, int64_t pos0, bool an
     const ps_seq_desc &D = m->d;
     const int64_t W = D.width;
     const bool tiled = (m->mode & 2) != 0;
-    psk_embed(st, D.embed, from_step ? nullptr : m->tokens, m->step, T, m->embed_scale, m->x, W);
+    const int64_t BW = (int64_t)D.max_batch * W;
+    psk_embed(st, D.embed, from_step ? nullptr : m->tokens, m->step, T, m->embed_scale, m->hist ? m->hist : m->x, W);
     auto mm = [&](const ps_dense *w, const float *a, int64_t lda, float *out, int64_t ldo) {
         psk_dense_args g;
         g.w = w; g.a = a; g.lda = lda; g.T = T; g.out = out; g.ldo = ldo; g.force_tiled = tiled; g.pack = m->pack; g.pack_bytes = m->pack_bytes;
@@ -380,13 +428,13 @@ static void seq_layers(ps_hip_seq *m, float *state, int T, int64_t pos0, bool an
     };
     // a sublayer boundary: x += norm_b(y) (after a sublayer), then hn = norm(x), h = conv(hn) (in front of the next one); one launch for a single token
     auto boundary = [&](const float *y, const float *wb, const float *wn, const float *cw, int64_t tail_off) {
-        if (T == 1 && !tiled) {
+        if (T == 1 && !tiled && m->groups == 1) {
             psk_boundary1(st, m->step, m->x, y, wb, wn, cw, D.canon_taps, tail_off, D.norm_offset, D.norm_eps, W, m->h, m->hn);
             return;
         }
-        if (y) psk_norm_residual(st, m->x, y, wb, D.norm_offset, D.norm_eps, W, T);
+        if (y) psk_norm_residual(st, m->x, y, wb, D.norm_offset, D.norm_eps, W, T, m->groups);
         if (wn) {
-            psk_rmsnorm(st, m->x, W, nullptr, wn, D.norm_offset, D.norm_eps, W, T, m->hn, W);
+            psk_rmsnorm(st, m->x, W, nullptr, wn, D.norm_offset, D.norm_eps, W, T, m->hn, W, m->groups);
             psk_causal_conv(st, m->step, tail_off, m->hn, W, cw, D.canon_taps, 0, W, T, m->h, W);
         }
     };
@@ -448,19 +496,28 @@ static void seq_layers(ps_hip_seq *m, float *state, int T, int64_t pos0, bool an
                 psk_dense(st, g);
             }
             psk_winattn_prep(st, m->step, P.off_ring, P.cap, P.off_pool, l.pool, t1, ld1, l.qnorm, l.knorm, D.norm_eps, (int)H, (int)G, (int)d, (int)dv, l.rot_dims,
-                             l.rot_pairing, P.freq, T, m->t2, Hd);
+                             l.rot_pairing, P.freq, T, m->t2, Hd, l.qtemp_coef, l.qtemp_every);
             const float *gate = l.gated ? t1 + Hd + G * d + G * dv : nullptr;
             const bool mfma = (m->mode & 2) == 0 && (G * (d + dv)) % 4 == 0 && psk_winattn_mfma_ok((int)d, (int)dv);
             if (mfma && T == 1 && m->win_scratch)
                 psk_winattn_step(st, m->step, P.off_ring, P.cap, P.off_pool, l.pool, m->t2, gate, l.temp, l.sink, (int)H, (int)G, (int)d, (int)dv, l.window, l.scale,
-                                 m->max_context, m->win_scratch, m->t3);
+                                 m->max_context, m->win_scratch, m->t3, l.softcap);
             else if (mfma)
                 psk_winattn_mfma(st, m->step, P.off_ring, P.cap, P.off_pool, l.pool, m->t2, Hd, gate, ld1, l.temp, l.sink, (int)H, (int)G, (int)d, (int)dv, l.window, l.scale,
-                                 T, m->t3, Hv);
+                                 T, m->t3, Hv, l.softcap);
             else
                 psk_winattn(st, m->step, P.off_ring, P.cap, P.off_pool, l.pool, m->t2, Hd, gate, ld1, l.temp, l.sink, (int)H, (int)G, (int)d, (int)dv, l.window, l.scale, T,
-                            m->t3, Hv);
+                            m->t3, Hv, l.softcap);
             out_proj(m->t3, Hv);
+        } else if (l.kind == PS_MIX_MINGRU) {
+            // t1 = [ z | x | g ] (+ bias); the recurrence and the gate -> t3; out
+            if (!P.in_ld) {
+                auto g = mm(l.in_cat, m->h, W, t1, ld1);
+                g.bias = l.in_bias;
+                psk_dense(st, g);
+            }
+            psk_mingru_scan(st, m->step, P.off_S, t1, ld1, d, T, m->t3, d);
+            out_proj(m->t3, d);
         } else {
             const int64_t dr = l.rot_dim, rs = l.kv_rank + dr, Hv = H * dv, nq = H * (d + dr);
             float *cq = m->t2, *q = m->t2 + (int64_t)D.max_batch * m->n_t2q;
@@ -500,24 +557,76 @@ static void seq_layers(ps_hip_seq *m, float *state, int T, int64_t pos0, bool an
         else { g.act = PSD_ACT_XIELU; g.act_p = P.act_p; g.act_q = P.act_q; }
         psk_dense(st, g);
     };
+    // The feed-forward of a parallel layer on `in`, added to xr times alpha.  Mixture of experts: slot s = t top + i is token t's i-th expert; the router's
+    // score scales what the expert READS (the A operand of its first product), a few tokens run grouped mat-vecs, a portion tiles over the slots sorted by expert.
+    auto feed_forward = [&](const LayerPlan &P, const float *in, float *xr, float alpha) {
+        const ps_seq_layer &l = P.d;
+        if (l.ff_kind != PS_FF_MOE_SWIGLU) {
+            ff_up(P, in);
+            auto g = mm(l.ff_down, m->t4, l.ff, xr, W);
+            g.accum = 1; g.alpha = alpha;
+            psk_dense(st, g);
+            return;
+        }
+        const int E = l.experts, top = l.top, S = T * top;
+        psk_moe_route(st, in, W, l.router, l.shared_gate, E, top, l.moe_norm_top, W, T, m->moe_sel, m->moe_wgt, m->moe_sg);
+        const bool mv = !tiled && T <= 8 && (size_t)std::max<int64_t>(W, (int64_t)top * l.ff) * 4 + 64 <= 128 * 1024;
+        if (!mv) psk_moe_plan(st, m->moe_sel, S, E, m->moe_seg, m->moe_list);
+        auto grouped = [&](psk_dense_args &g) {
+            g.groups = E; g.g_sel = m->moe_sel;
+            if (!mv) { g.g_seg = m->moe_seg; g.g_list = m->moe_list; }
+        };
+        {
+            auto g = mm(l.ff_up, in, W, m->t4, l.ff);
+            g.act = PSD_ACT_SILU_PAIR; g.T = S; g.g_adiv = top; g.g_scale = m->moe_wgt;
+            grouped(g);
+            psk_dense(st, g);
+        }
+        {
+            auto g = mm(l.ff_down, m->t4, l.ff, xr, W);
+            grouped(g);
+            if (mv) { g.T = T; g.g_inner = top; g.accum = 1; g.alpha = alpha; }
+            else if (top == 1) { g.T = S; g.accum = 1; g.alpha = alpha; }
+            else { g.T = S; g.out = m->moe_y; } // (two slots of a token sit in different tiles: per-slot results, summed below)
+            psk_dense(st, g);
+            if (!mv && top > 1) psk_moe_combine(st, xr, m->moe_y, top, alpha, W, T);
+        }
+        if (l.shared_up) {
+            auto g = mm(l.shared_up, in, W, m->t4, l.shared_ff);
+            g.act = PSD_ACT_SILU_PAIR;
+            psk_dense(st, g);
+            auto g2 = mm(l.shared_down, m->t4, l.shared_ff, xr, W);
+            g2.accum = 1; g2.alpha = alpha; g2.out_scale = l.shared_gate ? m->moe_sg : nullptr;
+            psk_dense(st, g2);
+        }
+    };
     const int n_runs = (int)m->L.size();
     if (m->L[0].d.form == PS_LAYER_SEQUENTIAL) boundary(nullptr, nullptr, m->L[0].d.norm1, m->L[0].d.canon1, m->L[0].off_canon1);
     for (int li = 0; li < n_runs; li++) {
         const LayerPlan &P = m->L[li];
         const ps_seq_layer &l = P.d;
         const LayerPlan *next = li + 1 < n_runs ? &m->L[li + 1] : nullptr;
-        if (l.form == PS_LAYER_PARALLEL) {
+        const float res = l.res_scale != 0.f ? l.res_scale : 1.f;
+        if (l.form == PS_LAYER_PARALLEL && !l.canon1) {
+            // No input filter: one launch makes the layer's input (with depth_mix: the previous layer's average over X_0 .. X_li, kept as this layer's X to add
+            // into) and both sublayers' norms; mixers and feed-forward add their output projections, times res, straight into the layer's X
+            float *xr = m->hist ? m->hist + (int64_t)(li + 1) * BW : m->x;
+            float *h2 = l.norm2 ? m->hn : nullptr;
+            if (m->hist) psk_front(st, m->hist, BW, li + 1, li ? m->L[li - 1].d.depth_mix : nullptr, nullptr, xr, l.norm1, m->h, l.norm2, h2, m->groups, D.norm_offset, D.norm_eps, W, T);
+            else psk_front(st, m->x, 0, 1, nullptr, nullptr, nullptr, l.norm1, m->h, l.norm2, h2, m->groups, D.norm_offset, D.norm_eps, W, T);
+            joint_in(P);
+            mixer(P, xr, res * l.mix_scale);
+            if (P.side) mixer(*P.side, xr, res * P.side->d.mix_scale);
+            if (l.ff_kind != PS_FF_NONE) feed_forward(P, h2 ? h2 : m->h, xr, res);
+            if (m->dbg_layers && !any_pos && m->hist)
+                psk_front(st, m->hist, BW, li + 2, l.depth_mix, nullptr, m->dbg_layers + (int64_t)li * BW, nullptr, nullptr, nullptr, nullptr, 1, 0.f, D.norm_eps, W, T);
+        } else if (l.form == PS_LAYER_PARALLEL) {
             // hn = norm(x), h = conv(hn); both mixers and the feed-forward add their output projections straight into the residual stream
             boundary(nullptr, nullptr, l.norm1, l.canon1, P.off_canon1);
             joint_in(P);
-            mixer(P, m->x, l.mix_scale);
-            if (P.side) mixer(*P.side, m->x, P.side->d.mix_scale);
-            if (l.ff_kind != PS_FF_NONE) {
-                ff_up(P, m->hn);
-                auto g = mm(l.ff_down, m->t4, l.ff, m->x, W);
-                g.accum = 1;
-                psk_dense(st, g);
-            }
+            mixer(P, m->x, res * l.mix_scale);
+            if (P.side) mixer(*P.side, m->x, res * P.side->d.mix_scale);
+            if (l.ff_kind != PS_FF_NONE) feed_forward(P, m->hn, m->x, res);
         } else {
             const bool summed = P.side != nullptr || l.mix_scale != 1.f;
             if (summed) psk_fill(st, m->y, 0.f, (int64_t)T * W);
@@ -536,7 +645,7 @@ static void seq_layers(ps_hip_seq *m, float *state, int T, int64_t pos0, bool an
                 boundary(m->y, l.norm1b, nn, nc, no);
             }
         }
-        if (m->dbg_layers && !any_pos) psk_copy(st, m->x, m->dbg_layers + (int64_t)li * D.max_batch * W, (int64_t)T * W);
+        if (m->dbg_layers && !any_pos && !m->hist) psk_copy(st, m->x, m->dbg_layers + (int64_t)li * BW, (int64_t)T * W);
     }
 }
 
@@ -544,7 +653,13 @@ static void seq_layers(ps_hip_seq *m, float *state, int T, int64_t pos0, bool an
 static void seq_head(ps_hip_seq *m, const int32_t *idx, int rows) {
     hipStream_t st = m->ctx->stream;
     const ps_seq_desc &D = m->d;
-    psk_rmsnorm(st, m->x, D.width, idx, D.final_norm, D.norm_offset, D.norm_eps, D.width, rows, m->xn, D.width);
+    if (m->hist) { // what the last layer hands on (its depth average, or its own result) and the final norm in one launch
+        const int runs = (int)m->L.size();
+        psk_front(st, m->hist, (int64_t)D.max_batch * D.width, runs + 1, m->L[runs - 1].d.depth_mix, idx, nullptr, D.final_norm, m->xn, nullptr, nullptr, m->groups,
+                  D.norm_offset, D.norm_eps, D.width, rows);
+    } else {
+        psk_rmsnorm(st, m->x, D.width, idx, D.final_norm, D.norm_offset, D.norm_eps, D.width, rows, m->xn, D.width, m->groups);
+    }
     psk_dense_args g;
     g.w = D.head; g.a = m->xn; g.lda = D.width; g.T = rows; g.out = m->logits; g.ldo = D.vocab; g.alpha = D.logit_scale; g.force_tiled = (m->mode & 2) != 0; g.pack = m->pack; g.pack_bytes = m->pack_bytes;
     psk_dense(st, g);

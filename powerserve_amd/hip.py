@@ -96,7 +96,10 @@ SeqLayer._fields_ = ([(n, C.c_int32) for n in ("kind", "heads", "kv_heads", "dim
                 [(n, C.c_void_p) for n in ("mu", "decay0", "bonus", "onorm", "conv", "a_log", "dt_bias", "qnorm", "kvnorm")] +
                 [("form", C.c_int32), ("mix_scale", C.c_float), ("beside", C.POINTER(SeqLayer))] +
                 [("pool", C.c_int32), ("rot_pairing", C.c_int32), ("gated", C.c_int32), ("rot_factor", C.c_float)] +
-                [(n, C.c_void_p) for n in ("in_bias", "knorm", "temp", "sink")] + [("tau", C.c_float)])
+                [(n, C.c_void_p) for n in ("in_bias", "knorm", "temp", "sink")] + [("tau", C.c_float)] +
+                [("res_scale", C.c_float), ("depth_mix", C.c_void_p), ("softcap", C.c_float), ("qtemp_coef", C.c_float), ("qtemp_every", C.c_int32)] +
+                [(n, C.c_int32) for n in ("experts", "top", "shared_ff", "moe_norm_top")] +
+                [(n, C.c_void_p) for n in ("router", "shared_gate", "shared_up", "shared_down")])
 
 
 class SeqDesc(C.Structure):
@@ -104,7 +107,7 @@ class SeqDesc(C.Structure):
     _fields_ = ([(n, C.c_int32) for n in ("n_layers", "width", "vocab", "canon_taps", "max_batch", "n_slots", "compute")] +
                 [("norm_eps", C.c_float), ("norm_offset", C.c_float), ("logit_scale", C.c_float)] +
                 [("embed", C.c_void_p), ("head", C.c_void_p), ("final_norm", C.c_void_p), ("layers", C.POINTER(SeqLayer))] +
-                [("embed_scale", C.c_float)] + [(n, C.c_int32) for n in ("loop_start", "loop_stop", "loop_times", "max_context")])
+                [("embed_scale", C.c_float)] + [(n, C.c_int32) for n in ("loop_start", "loop_stop", "loop_times", "max_context", "norm_groups")])
 
 
 _LIB = None

@@ -16,6 +16,16 @@ of layers that runs several times with the same weights (config 'loop'; every pa
                             a sink in the soft-max denominator, a temperature per head, RMS norms over the whole q / k projections, rotary on neighbouring
                             pairs of the first rot.dims numbers of a head with linearly scaled positions, a sigmoid gate per head;
                     right = gated linear attention (a decay per key channel from a two-matrix projection).
+
+Zusolix: PARALLEL layers with two norms of the same vector,  y = x + r * (mix(n1(x)) + mlp(n2(x))), RMS norms taken over 'norm.groups' equal parts of
+the vector, no input filter, a scaled embedding; what a layer hands on is a weighted average over the embedding and ALL layers' results so far (the layer's
+'dwa' weights).  Mixers:
+  attention         grouped-query soft-max attention over everything before the token, biases on q / k / v, no rotation; the query grows with the position
+                    (1 + coef ln(floor((p + 1) / every) + 1)), scores pass scale, then softcap * tanh(. / softcap)
+  mingru            an element-wise gated recurrence: z = sigmoid(W_z h + b), c = u + 1/2 (u >= 0) or sigmoid(u) with u = W_x h + b, S <- (1 - z) S + z c,
+                    output W_o (S * silu(W_g h))
+Feed-forward: SiLU-gated dense, or a mixture of such experts -- sigmoid router in fp32, the 'top' largest scores, a chosen expert's score multiplies its INPUT,
+plus a shared expert for every token times sigmoid of a one-row projection.
 """
 from __future__ import annotations
 
@@ -28,8 +38,8 @@ import numpy as np
 from . import hip
 from .safetensors_io import SafeTensors
 
-MIX_WKV, MIX_DELTA, MIX_LATENT, MIX_WINATTN, MIX_GLA = 1, 2, 3, 4, 5
-FF_NONE, FF_DENSE_XIELU, FF_DENSE_SWIGLU = 0, 1, 2
+MIX_WKV, MIX_DELTA, MIX_LATENT, MIX_WINATTN, MIX_GLA, MIX_MINGRU = 1, 2, 3, 4, 5, 6
+FF_NONE, FF_DENSE_XIELU, FF_DENSE_SWIGLU, FF_MOE_SWIGLU = 0, 1, 2, 3
 LAYER_SEQUENTIAL, LAYER_PARALLEL = 0, 1
 ROT_HALVES, ROT_NEIGHBOURS = 0, 1
 
@@ -118,6 +128,9 @@ def window_attention_mixer(L, st: SafeTensors, up, m: str, mc: dict, where: str)
     L.rot_dims, L.rot_base, L.rot_pairing = int(rot.get("dims") or 0), float(rot.get("base") or 10000.0), ROT_NEIGHBOURS
     L.rot_factor = float((rot.get("scaling") or {}).get("factor") or 1.0)
     L.scale = float(mc["scale"]) if mc.get("scale") is not None else L.dim ** -0.5
+    L.softcap = float(mc.get("softcap") or 0.0)
+    qt = mc.get("q_temp") or {}
+    L.qtemp_coef, L.qtemp_every = float(qt.get("coef") or 0.0), int(qt.get("every") or 0)
     rows = [(m + "q", L.heads * L.dim), (m + "k", L.kv_heads * L.dim), (m + "v", L.kv_heads * L.vdim)]
     L.gated = int(m + "g" in st)
     if L.gated:
@@ -153,6 +166,78 @@ def gated_linear_mixer(L, st: SafeTensors, up, m: str, mc: dict, where: str):
     L.decay0 = up.vec(_expect(st, m + "a2.b", (L.heads * L.dim,)) if m + "a2.b" in st else np.zeros(L.heads * L.dim, np.float32))
     L.onorm = up.vec(_expect(st, m + "norm", (L.vdim,)))
     L.out = up.mat(st.bf16_bits(m + "o"))
+
+
+def gated_recurrence_mixer(L, st: SafeTensors, up, m: str, mc: dict, where: str):
+    """Fill descriptor L with an element-wise gated recurrence (MIX_MINGRU): z | x | g stacked with one bias vector (zeros where a projection has none)."""
+    L.kind, L.heads = MIX_MINGRU, 1
+    L.dim = L.vdim = int(mc["width"])
+    for n in ("z", "x", "g"):
+        if st.shape(m + n)[0] != L.dim:
+            raise ConfigError(f"tensor {m + n}: {st.shape(m + n)[0]} rows, the configuration gives {L.dim} ({where})")
+    L.in_cat = up.mat(_stack(st, [m + n for n in ("z", "x", "g")]))
+    if any(m + n + ".b" in st for n in ("z", "x", "g")):
+        L.in_bias = up.vec(np.concatenate([_expect(st, m + n + ".b", (L.dim,)) if m + n + ".b" in st else np.zeros(L.dim, np.float32) for n in ("z", "x", "g")]))
+    L.out = up.mat(st.bf16_bits(m + "o"))
+
+
+def _gate_up(st: SafeTensors, p: str, ff: int, width: int, where: str) -> np.ndarray:
+    """rows gate_0, up_0, gate_1, ... of the feed-forward under prefix p: the pair meets in one epilogue"""
+    gate, upw = st.bf16_bits(p + "gate"), st.bf16_bits(p + "up")
+    if gate.shape != (ff, width) or upw.shape != (ff, width) or st.shape(p + "down") != (width, ff):
+        raise ConfigError(f"{where}: feed-forward shapes {gate.shape} / {upw.shape} / {st.shape(p + 'down')}, the configuration gives {(ff, width)}")
+    return np.stack([gate, upw], axis=1).reshape(2 * ff, width)
+
+
+def gated_feed_forward(L, st: SafeTensors, up, p: str, mlp: dict, width: int, where: str):
+    """Fill descriptor L's feed-forward from the tensors under prefix p: 'dense' (SiLU-gated) or 'moe' (experts e0, e1, ... of that form stacked into one
+    matrix each way, an fp32 router, an optional shared expert with an optional one-row gate)."""
+    kind = mlp.get("kind")
+    if kind == "dense":
+        L.ff_kind, L.ff = FF_DENSE_SWIGLU, int(mlp["ff"])
+        L.ff_up, L.ff_down = up.mat(_gate_up(st, p, L.ff, width, where)), up.mat(st.bf16_bits(p + "down"))
+    elif kind == "moe":
+        r = mlp["router"]
+        L.ff_kind, L.ff, L.experts, L.top = FF_MOE_SWIGLU, int(mlp["expert"]["ff"]), int(r["experts"]), int(r["top"])
+        if not 0 < L.top <= L.experts:
+            raise ConfigError(f"{where}: top {L.top} of {L.experts} experts")
+        L.ff_up = up.mat(np.concatenate([_gate_up(st, f"{p}e{e}.", L.ff, width, where) for e in range(L.experts)], axis=0))
+        L.ff_down = up.mat(np.concatenate([st.bf16_bits(f"{p}e{e}.down") for e in range(L.experts)], axis=0))
+        L.router = up.vec(_expect(st, p + "router", (L.experts, width)))
+        if mlp.get("shared"):
+            L.shared_ff = int(mlp["shared"]["ff"])
+            L.shared_up, L.shared_down = up.mat(_gate_up(st, p + "shared.", L.shared_ff, width, where)), up.mat(st.bf16_bits(p + "shared.down"))
+            if p + "shared.sg" in st:
+                L.shared_gate = up.vec(_expect(st, p + "shared.sg", (1, width)).reshape(-1))
+    else:
+        raise ConfigError(f"{where}: feed-forward kind {kind!r} is not known")
+
+
+def _zusolix_layers(cfg: dict, st: SafeTensors, up) -> tuple[list, dict]:
+    width = int(cfg["width"])
+    layers = []
+    for i, lc in enumerate(cfg["layers"]):
+        p, mc, kind = f"l{i}.", lc["mixer"], lc["type"]
+        L = hip.SeqLayer()
+        L.form, L.mix_scale, L.res_scale = LAYER_PARALLEL, 1.0, float(cfg.get("residual_mult") or 1.0)
+        L.norm1 = up.vec(_expect(st, p + "norm1", (width,)))
+        if kind == "attention":
+            window_attention_mixer(L, st, up, p + "mix.", mc, f"layer {i}")
+        elif kind == "mingru":
+            gated_recurrence_mixer(L, st, up, p + "mix.", mc, f"layer {i}")
+        else:
+            raise ConfigError(f"layer {i}: mixer type {kind!r} is not known")
+        if lc.get("mlp"):
+            L.norm2 = up.vec(_expect(st, p + "norm2", (width,)))
+            gated_feed_forward(L, st, up, p + "mlp.", lc["mlp"], width, f"layer {i}")
+        if p + "dwa" in st:
+            L.depth_mix = up.vec(_expect(st, p + "dwa", (i + 2,)))
+        layers.append(L)
+    norm = cfg.get("norm") or {}
+    top = dict(width=width, vocab=int(cfg["vocab"]), canon_taps=1, norm_eps=float(norm["eps"]), norm_groups=int(norm.get("groups") or 1), norm_offset=0.0,
+               logit_scale=1.0, embed_scale=float((cfg.get("embedding") or {}).get("scale") or 1.0), embed=up.mat(st.bf16_bits("embed")),
+               head=up.mat(st.bf16_bits("head")), final_norm=up.vec(_expect(st, "final.norm", (width,))))
+    return layers, top
 
 
 def _vobisun_layers(cfg: dict, st: SafeTensors, up) -> tuple[list, dict]:
@@ -194,7 +279,7 @@ def _vobisun_layers(cfg: dict, st: SafeTensors, up) -> tuple[list, dict]:
     return layers, top
 
 
-ARCHITECTURES = {"Ranutar": _ranutar_layers, "Vobisun": _vobisun_layers}
+ARCHITECTURES = {"Ranutar": _ranutar_layers, "Vobisun": _vobisun_layers, "Zusolix": _zusolix_layers}
 
 
 def read_config(model_dir: str) -> dict:
