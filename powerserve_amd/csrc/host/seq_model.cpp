@@ -215,6 +215,8 @@ void window_attention_mixer(ps_seq_layer &L, const SafeTensorsFile &st, SeqUploa
         if (const JsonValue *sc = obj_or_null(*rot, "scaling")) L.rot_factor = (float)num_or(*sc, "factor", 1.0);
     }
     L.scale = (float)num_or(mc, "scale", 1.0 / std::sqrt((double)L.dim));
+    L.softcap = (float)num_or(mc, "softcap", 0.0);
+    if (const JsonValue *qt = obj_or_null(mc, "q_temp")) { L.qtemp_coef = (float)num_or(*qt, "coef", 0.0); L.qtemp_every = (int32_t)num_or(*qt, "every", 0); }
     L.gated = st.contains(m + "g") ? 1 : 0;
     std::vector<std::pair<std::string, int64_t>> rows = {{m + "q", (int64_t)L.heads * L.dim}, {m + "k", (int64_t)L.kv_heads * L.dim}, {m + "v", (int64_t)L.kv_heads * L.vdim}};
     if (L.gated) rows.push_back({m + "g", L.heads});
@@ -306,10 +308,112 @@ void vobisun(const JsonValue &cfg, const SafeTensorsFile &st, SeqUploader &up, s
         layers.push_back(L);
     }
 }
+
+// ---------------------------------------------------------------- Zusolix: two-norm parallel layers, depth average, attention / gated recurrence, dense / expert feed-forwards
+void gated_recurrence_mixer(ps_seq_layer &L, const SafeTensorsFile &st, SeqUploader &up, const std::string &m, const JsonValue &mc) {
+    L.kind = PS_MIX_MINGRU;
+    L.heads = 1;
+    L.dim = L.vdim = (int32_t)mc.at("width").num;
+    std::vector<std::string> names;
+    std::vector<float> bias;
+    bool any_bias = false;
+    for (const char *n : {"z", "x", "g"}) {
+        if (rows_of(st, m + n) != L.dim) POWERSERVE_ABORT("tensor " + m + n + ": its rows are not what the configuration gives");
+        names.push_back(m + n);
+        if (st.contains(m + n + ".b")) { auto b = expect1(st, m + n + ".b", L.dim); bias.insert(bias.end(), b.begin(), b.end()); any_bias = true; }
+        else bias.insert(bias.end(), (size_t)L.dim, 0.f);
+    }
+    L.in_cat = mat_rows(st, up, names);
+    if (any_bias) L.in_bias = up.vec(bias);
+    L.out = mat1(st, up, m + "o");
+}
+// rows gate_0, up_0, gate_1, ... of the feed-forward under prefix p appended to `all`: the pair meets in one epilogue
+void append_gate_up(const SafeTensorsFile &st, const std::string &p, int64_t ff, int64_t W, std::vector<uint16_t> &all) {
+    const auto g = st.bf16_bits(p + "gate"), u = st.bf16_bits(p + "up");
+    if ((int64_t)g.size() != ff * W || u.size() != g.size() || rows_of(st, p + "down") != W || cols_of(st, p + "down") != ff) POWERSERVE_ABORT(p + ": feed-forward shapes");
+    const size_t at = all.size();
+    all.resize(at + 2 * g.size());
+    for (int64_t r = 0; r < ff; r++) {
+        memcpy(&all[at + (size_t)(2 * r) * W], &g[(size_t)r * W], (size_t)W * 2);
+        memcpy(&all[at + (size_t)(2 * r + 1) * W], &u[(size_t)r * W], (size_t)W * 2);
+    }
+}
+void gated_feed_forward(ps_seq_layer &L, const SafeTensorsFile &st, SeqUploader &up, const std::string &p, const JsonValue &f, int64_t W) {
+    const std::string kind = f.at("kind").str;
+    if (kind == "dense") {
+        L.ff_kind = PS_FF_DENSE_SWIGLU;
+        L.ff = (int32_t)f.at("ff").num;
+        std::vector<uint16_t> both;
+        append_gate_up(st, p, L.ff, W, both);
+        L.ff_up = up.mat(both, 2 * (int64_t)L.ff, W);
+        L.ff_down = mat1(st, up, p + "down");
+    } else if (kind == "moe") {
+        L.ff_kind = PS_FF_MOE_SWIGLU;
+        L.ff = (int32_t)f.at("expert").at("ff").num;
+        L.experts = (int32_t)f.at("router").at("experts").num;
+        L.top = (int32_t)f.at("router").at("top").num;
+        if (L.experts <= 0 || L.top <= 0 || L.top > L.experts) POWERSERVE_ABORT(p + ": top / experts");
+        std::vector<uint16_t> ups, downs;
+        for (int e = 0; e < L.experts; e++) {
+            const std::string pe = p + "e" + std::to_string(e) + ".";
+            append_gate_up(st, pe, L.ff, W, ups);
+            const auto dn = st.bf16_bits(pe + "down");
+            downs.insert(downs.end(), dn.begin(), dn.end());
+        }
+        L.ff_up = up.mat(ups, (int64_t)L.experts * 2 * L.ff, W);
+        L.ff_down = up.mat(downs, (int64_t)L.experts * W, L.ff);
+        L.router = up.vec(expect(st, p + "router", L.experts, W));
+        if (const JsonValue *sh = obj_or_null(f, "shared")) {
+            L.shared_ff = (int32_t)sh->at("ff").num;
+            std::vector<uint16_t> both;
+            append_gate_up(st, p + "shared.", L.shared_ff, W, both);
+            L.shared_up = up.mat(both, 2 * (int64_t)L.shared_ff, W);
+            L.shared_down = mat1(st, up, p + "shared.down");
+            if (st.contains(p + "shared.sg")) L.shared_gate = up.vec(expect(st, p + "shared.sg", 1, W));
+        }
+    } else {
+        POWERSERVE_ABORT(p + ": feed-forward kind " + kind + " is not known");
+    }
+}
+void zusolix(const JsonValue &cfg, const SafeTensorsFile &st, SeqUploader &up, std::vector<ps_seq_layer> &layers, ps_seq_desc &d) {
+    d.width = (int32_t)cfg.at("width").num;
+    d.vocab = (int32_t)cfg.at("vocab").num;
+    d.canon_taps = 1;
+    d.norm_eps = (float)cfg.at("norm").at("eps").num;
+    d.norm_groups = (int32_t)num_or(cfg.at("norm"), "groups", 1);
+    d.norm_offset = 0.0f;
+    d.logit_scale = 1.0f;
+    d.loop_times = 1;
+    const JsonValue *emb = obj_or_null(cfg, "embedding");
+    d.embed_scale = emb ? (float)num_or(*emb, "scale", 1.0) : 1.0f;
+    const float res = (float)num_or(cfg, "residual_mult", 1.0);
+    d.embed = mat1(st, up, "embed");
+    d.head = mat1(st, up, "head");
+    d.final_norm = up.vec(expect1(st, "final.norm", d.width));
+    const auto &ls = cfg.at("layers").arr;
+    for (size_t i = 0; i < ls.size(); i++) {
+        const JsonValue &lc = ls[i], &mc = lc.at("mixer");
+        const std::string p = "l" + std::to_string(i) + ".", kind = lc.at("type").str;
+        ps_seq_layer L{};
+        L.form = PS_LAYER_PARALLEL;
+        L.mix_scale = 1.f;
+        L.res_scale = res;
+        L.norm1 = up.vec(expect1(st, p + "norm1", d.width));
+        if (kind == "attention") window_attention_mixer(L, st, up, p + "mix.", mc);
+        else if (kind == "mingru") gated_recurrence_mixer(L, st, up, p + "mix.", mc);
+        else POWERSERVE_ABORT("layer " + std::to_string(i) + ": mixer type " + kind + " is not known");
+        if (lc.contains("mlp") && lc.at("mlp").kind == JsonValue::OBJ) {
+            L.norm2 = up.vec(expect1(st, p + "norm2", d.width));
+            gated_feed_forward(L, st, up, p + "mlp.", lc.at("mlp"), d.width);
+        }
+        if (st.contains(p + "dwa")) L.depth_mix = up.vec(expect1(st, p + "dwa", (int64_t)i + 2));
+        layers.push_back(L);
+    }
+}
 } // namespace
 
 const std::map<std::string, SeqArchitecture> &seq_architectures() {
-    static const std::map<std::string, SeqArchitecture> reg = {{"Ranutar", ranutar}, {"Vobisun", vobisun}};
+    static const std::map<std::string, SeqArchitecture> reg = {{"Ranutar", ranutar}, {"Vobisun", vobisun}, {"Zusolix", zusolix}};
     return reg;
 }
 bool is_seq_model_dir(const std::string &dir) {

@@ -277,11 +277,88 @@ def _parallel_tensors(cfg: dict, seed: int, decay_rank: int) -> dict:
     return t
 
 
+def zusolix_attention(heads: int, kv_heads: int, dim: int, vdim: int, scale: float, softcap: float | None = None, q_temp: tuple | None = None) -> dict:
+    """mixer entry of a Zusolix attention layer; q_temp: (coef, every) or None"""
+    mc = {"heads": int(heads), "kv_heads": int(kv_heads), "dim": int(dim), "vdim": int(vdim), "scale": float(scale)}
+    if softcap:
+        mc["softcap"] = float(softcap)
+    if q_temp:
+        mc["q_temp"] = {"coef": float(q_temp[0]), "every": int(q_temp[1])}
+    return mc
+
+
+def zusolix_layer(kind: str, mixer: dict, ff: int | None = None, moe: tuple | None = None, shared: int | None = None) -> dict:
+    """One entry of a Zusolix configuration's 'layers'.  kind 'attention' (mixer: zusolix_attention) or 'mingru' (mixer: {'width': n}); the feed-forward
+    is dense (ff), a mixture (moe = (experts, top, expert ff), shared = the shared expert's ff or None), or absent."""
+    mlp = None
+    if moe:
+        mlp = {"kind": "moe", "router": {"experts": int(moe[0]), "top": int(moe[1])}, "expert": {"ff": int(moe[2])}}
+        if shared:
+            mlp["shared"] = {"ff": int(shared)}
+    elif ff:
+        mlp = {"kind": "dense", "ff": int(ff)}
+    return {"type": kind, "mixer": dict(mixer), "mlp": mlp}
+
+
+def zusolix_config(width: int, vocab: int, layers: list, groups: int = 1, eps: float = 1e-6, embed_scale: float = 1.0, residual_mult: float = 1.0) -> dict:
+    return {"architecture": "Zusolix", "embedding": {"scale": float(embed_scale)}, "layers": layers, "norm": {"eps": float(eps), "groups": int(groups)},
+            "residual_mult": float(residual_mult), "vocab": int(vocab), "width": int(width)}
+
+
+def _zusolix_tensors(cfg: dict, seed: int) -> dict:
+    rng = np.random.default_rng(seed)
+    W = cfg["width"]
+
+    def lin(n, k, gain=1.0):
+        return rng.standard_normal((n, k), dtype=np.float32) * np.float32(gain / np.sqrt(k))
+
+    def vec(n, std=0.1, mean=0.0):
+        return (rng.standard_normal(n, dtype=np.float32) * np.float32(std) + np.float32(mean)).astype(np.float32)
+
+    def ffn(p, ff):
+        t[p + "gate"], t[p + "up"], t[p + "down"] = lin(ff, W), lin(ff, W), lin(W, ff)
+
+    t = {"embed": rng.standard_normal((cfg["vocab"], W), dtype=np.float32) / np.float32(cfg["embedding"]["scale"])}
+    for i, lc in enumerate(cfg["layers"]):
+        p, m, mc = f"l{i}.", f"l{i}.mix.", lc["mixer"]
+        t[p + "norm1"] = vec(W, 0.2, 1.0)
+        if lc["type"] == "attention":
+            H, G, d, dv = mc["heads"], mc["kv_heads"], mc["dim"], mc["vdim"]
+            for n, rows in (("q", H * d), ("k", G * d), ("v", G * dv)):
+                t[m + n], t[m + n + ".b"] = lin(rows, W, 1.5), vec(rows, 0.3)
+            t[m + "o"] = lin(W, H * dv)
+        elif lc["type"] == "mingru":
+            C = mc["width"]
+            for n in ("z", "x"):
+                t[m + n], t[m + n + ".b"] = lin(C, W, 1.5), vec(C, 0.5)
+            t[m + "g"], t[m + "o"] = lin(C, W), lin(W, C)
+        else:
+            raise ValueError(lc["type"])
+        mlp = lc.get("mlp")
+        if mlp:
+            t[p + "norm2"] = vec(W, 0.2, 1.0)
+            if mlp["kind"] == "dense":
+                ffn(p + "mlp.", mlp["ff"])
+            else:
+                for e in range(mlp["router"]["experts"]):
+                    ffn(f"{p}mlp.e{e}.", mlp["expert"]["ff"])
+                t[p + "mlp.router"] = lin(mlp["router"]["experts"], W, 2.0)
+                if mlp.get("shared"):
+                    ffn(p + "mlp.shared.", mlp["shared"]["ff"])
+                    t[p + "mlp.shared.sg"] = lin(1, W, 2.0)
+        # the weights of the depth average: mostly the layer's own result, the rest spread (with signs) over everything before it
+        w = rng.standard_normal(i + 2).astype(np.float32) * np.float32(0.2)
+        w[-1] += 1.0
+        t[p + "dwa"] = w
+    t["final.norm"], t["head"] = vec(W, 0.2, 1.0), lin(cfg["vocab"], W)
+    return t
+
+
 def seq_tensors(cfg: dict, seed: int = 0, decay_rank: int = 8) -> dict:
     """Random-init tensors of a layer-list configuration, name -> float32 array already rounded to bfloat16 (what the file will hold)."""
     from .safetensors_io import f32_to_bf16_bits
-    if cfg.get("architecture") == "Vobisun":
-        t = _parallel_tensors(cfg, seed, decay_rank)
+    if cfg.get("architecture") in ("Vobisun", "Zusolix"):
+        t = _parallel_tensors(cfg, seed, decay_rank) if cfg["architecture"] == "Vobisun" else _zusolix_tensors(cfg, seed)
         return {k: (f32_to_bf16_bits(v).astype(np.uint32) << 16).view(np.float32).reshape(v.shape) for k, v in t.items()}
     rng = np.random.default_rng(seed)
     W, taps = cfg["width"], cfg["canon"]["taps"]

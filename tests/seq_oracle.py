@@ -288,3 +288,121 @@ def run_parallel(cfg, W, tokens, per_layer=None, **kw):
         if per_layer is not None:
             per_layer.append(x.copy())
     return plain_norm(x, W["final.norm"], eps) @ W["head"].T
+
+
+# ---------------------------------------------------------------------------------------------------------------- Zusolix
+# Parallel layers with two norms of the same vector,  X_(i+1) = x_i + m (mixer(norm1(x_i)) + ff(norm2(x_i))), where x_i, the input of layer i, is a
+# weighted average over the embedding X_0 and all earlier results X_1 .. X_i (x_0 = X_0); norms in groups; attention without rotation whose queries
+# grow with the position and whose scores are soft-capped; an element-wise gated recurrence; dense or mixture-of-experts feed-forwards.
+def sigmoid(a):
+    return 1.0 / (1.0 + np.exp(-a))
+
+
+def grouped_norm(a, w, groups, eps):
+    """the vector in `groups` equal consecutive parts, each divided by the root of (its own mean square + eps); then the weight"""
+    n = a.shape[-1] // groups
+    out = np.empty_like(a)
+    for g in range(groups):
+        part = a[..., g * n:(g + 1) * n]
+        out[..., g * n:(g + 1) * n] = part / np.sqrt(np.mean(part * part, axis=-1, keepdims=True) + eps)
+    return out * w
+
+
+def query_temperature(p, coef, every):
+    return 1.0 + coef * np.log(np.floor((p + 1) / every) + 1.0)
+
+
+def capped_attention(W, pre, h, mc, reach=None, use_cap=True, use_temperature=True, temperature_shift=0):
+    """Causal grouped-query soft-max attention, biases on q / k / v, no rotation.  reach: a WRONG model on purpose, in which a query sees only the last
+    `reach` positions; use_cap / use_temperature False: wrong models without the soft cap / the query temperature; temperature_shift: a wrong model whose
+    temperature steps that many tokens late (negative: early)."""
+    T = h.shape[0]
+    H, G, d, dv = mc["heads"], mc.get("kv_heads", mc["heads"]), mc["dim"], mc.get("vdim", mc["dim"])
+    out = np.zeros((T, H * dv))
+    keys, values = [], []
+    cap, qt = mc.get("softcap"), mc.get("q_temp")
+    for t in range(T):
+        q = (W[pre + "q"] @ h[t] + W[pre + "q.b"]).reshape(H, d)
+        keys.append((W[pre + "k"] @ h[t] + W[pre + "k.b"]).reshape(G, d))
+        values.append((W[pre + "v"] @ h[t] + W[pre + "v.b"]).reshape(G, dv))
+        if qt and use_temperature:
+            q = q * query_temperature(max(0, t - temperature_shift), qt["coef"], qt["every"])
+        first = 0 if reach is None else max(0, t - reach + 1)
+        for hd in range(H):
+            g = hd // (H // G)
+            s = np.array([q[hd] @ keys[j][g] for j in range(first, t + 1)]) * mc["scale"]
+            if cap and use_cap:
+                s = cap * np.tanh(s / cap)
+            e = np.exp(s - s.max())
+            a = e / e.sum()
+            out[t, hd * dv:(hd + 1) * dv] = sum(a[j - first] * values[j][g] for j in range(first, t + 1))
+    return out @ W[pre + "o"].T
+
+
+def min_gru(W, pre, h, mc, carry=True):
+    """carry False: a WRONG model in which the state is lost at every token"""
+    C = mc["width"]
+    S = np.zeros(C)
+    out = np.zeros((h.shape[0], C))
+    for t in range(h.shape[0]):
+        z = sigmoid(W[pre + "z"] @ h[t] + W[pre + "z.b"])
+        u = W[pre + "x"] @ h[t] + W[pre + "x.b"]
+        cand = np.where(u >= 0, u + 0.5, sigmoid(u))
+        S = (1.0 - z) * (S if carry else 0.0) + z * cand
+        out[t] = S * silu(W[pre + "g"] @ h[t])
+    return out @ W[pre + "o"].T
+
+
+def one_expert(W, pre, a):
+    return W[pre + "down"] @ (silu(W[pre + "gate"] @ a) * (W[pre + "up"] @ a))
+
+
+def expert_mixture(W, pre, h, mlp, weight_on_output=False, use_shared=True):
+    """Scores sigmoid(router h); the `top` largest (the lower index on a tie); a chosen expert sees score * h.  weight_on_output: a WRONG model in which
+    the score multiplies the expert's result instead."""
+    E, top = mlp["router"]["experts"], mlp["router"]["top"]
+    out = np.zeros_like(h)
+    for t in range(h.shape[0]):
+        s = sigmoid(W[pre + "router"] @ h[t])
+        left = list(range(E))
+        for _ in range(top):
+            e = max(left, key=lambda i: (s[i], -i))
+            left.remove(e)
+            out[t] += s[e] * one_expert(W, f"{pre}e{e}.", h[t]) if weight_on_output else one_expert(W, f"{pre}e{e}.", s[e] * h[t])
+        if mlp.get("shared") and use_shared:
+            gate = sigmoid(W[pre + "shared.sg"] @ h[t])[0] if pre + "shared.sg" in W else 1.0
+            out[t] += gate * one_expert(W, pre + "shared.", h[t])
+    return out
+
+
+def zusolix_feed_forward(W, pre, h, mlp, **kw):
+    if mlp["kind"] == "dense":
+        return np.stack([one_expert(W, pre, h[t]) for t in range(h.shape[0])])
+    return expert_mixture(W, pre, h, mlp, **kw)
+
+
+def depth_average(w, streams):
+    return sum(w[j] * streams[j] for j in range(len(streams)))
+
+
+def run_zusolix(cfg, W, tokens, per_layer=None, use_depth=True, attn_kw=None, gru_kw=None, moe_kw=None):
+    """-> logits [T, vocab]; per_layer (a list) receives what every layer hands on.  use_depth False: a WRONG model without the depth average."""
+    W = {k: np.asarray(v, dtype=np.float64) for k, v in W.items()}
+    eps, groups, m = cfg["norm"]["eps"], cfg["norm"].get("groups", 1), cfg.get("residual_mult", 1.0)
+    x = W["embed"][np.asarray(tokens)] * cfg.get("embedding", {}).get("scale", 1.0)
+    streams = [x]
+    for i, lc in enumerate(cfg["layers"]):
+        p = f"l{i}."
+        h1 = grouped_norm(x, W[p + "norm1"], groups, eps)
+        if lc["type"] == "attention":
+            y = capped_attention(W, p + "mix.", h1, lc["mixer"], **(attn_kw or {}))
+        else:
+            y = min_gru(W, p + "mix.", h1, lc["mixer"], **(gru_kw or {}))
+        if lc.get("mlp"):
+            kw = (moe_kw or {}) if lc["mlp"]["kind"] == "moe" else {}
+            y = y + zusolix_feed_forward(W, p + "mlp.", grouped_norm(x, W[p + "norm2"], groups, eps), lc["mlp"], **kw)
+        streams.append(x + m * y)
+        x = depth_average(W[p + "dwa"], streams) if use_depth and p + "dwa" in W else streams[-1]
+        if per_layer is not None:
+            per_layer.append(x)
+    return grouped_norm(x, W["final.norm"], groups, eps) @ W["head"].T

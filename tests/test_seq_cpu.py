@@ -89,13 +89,17 @@ def test_ctypes_descriptors_match_the_header(tmp_path):
     src.write_text('#include <stdio.h>\n#include <stddef.h>\n#include "ps_hip.h"\nint main(void){printf("%zu %zu %zu %zu %zu %zu %zu %zu %zu %zu %zu\\n", sizeof(ps_seq_layer), '
                    'offsetof(ps_seq_layer, norm1), offsetof(ps_seq_layer, kvnorm), sizeof(ps_seq_desc), offsetof(ps_seq_desc, embed), offsetof(ps_seq_desc, layers), '
                    'offsetof(ps_seq_layer, beside), offsetof(ps_seq_layer, in_bias), offsetof(ps_seq_layer, tau), offsetof(ps_seq_desc, embed_scale), '
-                   'offsetof(ps_seq_desc, max_context));return 0;}\n')
+                   'offsetof(ps_seq_desc, max_context));'
+                   'printf("%zu %zu %zu %zu %zu %zu %zu\\n", offsetof(ps_seq_layer, res_scale), offsetof(ps_seq_layer, depth_mix), offsetof(ps_seq_layer, softcap), '
+                   'offsetof(ps_seq_layer, qtemp_every), offsetof(ps_seq_layer, experts), offsetof(ps_seq_layer, shared_down), offsetof(ps_seq_desc, norm_groups));return 0;}\n')
     exe = str(tmp_path / "sz")
     subprocess.run(["gcc", "-I" + os.path.join(ROOT, "include"), str(src), "-o", exe], check=True)
     got = [int(x) for x in subprocess.run([exe], check=True, capture_output=True, text=True).stdout.split()]
     assert got == [C.sizeof(hip.SeqLayer), hip.SeqLayer.norm1.offset, hip.SeqLayer.kvnorm.offset, C.sizeof(hip.SeqDesc), hip.SeqDesc.embed.offset,
                    hip.SeqDesc.layers.offset, hip.SeqLayer.beside.offset, hip.SeqLayer.in_bias.offset, hip.SeqLayer.tau.offset, hip.SeqDesc.embed_scale.offset,
-                   hip.SeqDesc.max_context.offset]
+                   hip.SeqDesc.max_context.offset,
+                   hip.SeqLayer.res_scale.offset, hip.SeqLayer.depth_mix.offset, hip.SeqLayer.softcap.offset, hip.SeqLayer.qtemp_every.offset, hip.SeqLayer.experts.offset,
+                   hip.SeqLayer.shared_down.offset, hip.SeqDesc.norm_groups.offset]
 
 
 def test_plain_statement_is_causal_and_windowed():
@@ -178,6 +182,85 @@ def test_plain_parallel_statement_reach():
     assert changed == [7, 8, 9, 10, 11] + list(range(13, 24))
     la, lb = seq_oracle.run_parallel(one, t, a, pool=0), seq_oracle.run_parallel(one, t, b, pool=0)
     assert [i for i in range(24) if np.abs(la[i] - lb[i]).max() > 1e-9] == [7, 8, 9, 10, 11]
+
+
+ZCFG = synth.zusolix_config(24, 30, [
+    synth.zusolix_layer("attention", synth.zusolix_attention(4, 2, 6, 10, 0.25, 7.0, (0.3, 9)), moe=(3, 2, 8), shared=5),
+    synth.zusolix_layer("mingru", {"width": 14}, ff=20),
+    synth.zusolix_layer("attention", synth.zusolix_attention(2, 2, 6, 6, 0.5))], groups=3, eps=1e-5, embed_scale=3.0, residual_mult=0.4)
+
+
+def test_zusolix_configuration_maps_onto_layer_descriptors(tmp_path):
+    t = synth.write_seq_model_dir(str(tmp_path), ZCFG, 1)
+    cfg = seqmodel.read_config(str(tmp_path))
+    up = FakeUp()
+    st = safetensors_io.SafeTensors(str(tmp_path / "model.safetensors"))
+    layers, top = seqmodel.ARCHITECTURES[cfg["architecture"]](cfg, st, up)
+    bits = safetensors_io.f32_to_bf16_bits
+    assert (top["width"], top["vocab"], top["canon_taps"], top["norm_offset"], top["embed_scale"], top["norm_groups"]) == (24, 30, 1, 0.0, 3.0, 3)
+    a, g, c = layers
+    assert all(abs(x.res_scale - 0.4) < 1e-7 and x.form == seqmodel.LAYER_PARALLEL and x.canon1 is None for x in layers)
+    assert (a.kind, a.heads, a.kv_heads, a.dim, a.vdim, a.window, a.pool, a.rot_dims, a.gated, a.qtemp_every) == (seqmodel.MIX_WINATTN, 4, 2, 6, 10, 0, 0, 0, 0, 9)
+    assert abs(a.softcap - 7.0) < 1e-6 and abs(a.qtemp_coef - 0.3) < 1e-6 and a.scale == 0.25 and (c.softcap, c.qtemp_every, c.qtemp_coef) == (0.0, 0, 0.0)
+    assert (a.qnorm, a.knorm, a.temp, a.sink) == (None, None, None, None)
+    bias = up.vecs[a.in_bias - 1]
+    assert bias.shape == (24 + 12 + 20,) and np.array_equal(bias[24:36], t["l0.mix.k.b"])
+    # the depth average's weights: one more per layer
+    assert [up.vecs[x.depth_mix - 1].shape for x in layers] == [(2,), (3,), (4,)] and a.norm2 is not None and c.norm2 is None and c.ff_kind == seqmodel.FF_NONE
+    # the recurrence: z | x | g stacked, one bias vector (g has none)
+    assert (g.kind, g.heads, g.dim, g.ff_kind, g.ff) == (seqmodel.MIX_MINGRU, 1, 14, seqmodel.FF_DENSE_SWIGLU, 20)
+    assert np.array_equal(up.mats[g.in_cat - 1001], np.concatenate([bits(t["l1.mix." + n]) for n in ("z", "x", "g")]))
+    gb = up.vecs[g.in_bias - 1]
+    assert gb.shape == (42,) and np.array_equal(gb[14:28], t["l1.mix.x.b"]) and not gb[28:].any()
+    # the experts: one matrix each way, expert after expert, gate / up rows alternating inside an expert; the router and the shared gate stay fp32 vectors
+    assert (a.ff_kind, a.ff, a.experts, a.top, a.shared_ff, a.moe_norm_top) == (seqmodel.FF_MOE_SWIGLU, 8, 3, 2, 5, 0)
+    ups, downs = up.mats[a.ff_up - 1001], up.mats[a.ff_down - 1001]
+    assert ups.shape == (3 * 16, 24) and downs.shape == (3 * 24, 8)
+    assert np.array_equal(ups[16:32:2], bits(t["l0.mlp.e1.gate"])) and np.array_equal(ups[33:48:2], bits(t["l0.mlp.e2.up"])) and np.array_equal(downs[24:48], bits(t["l0.mlp.e1.down"]))
+    assert up.vecs[a.router - 1].shape == (3, 24) and up.vecs[a.shared_gate - 1].shape == (24,) and up.mats[a.shared_up - 1001].shape == (10, 24)
+    # what the file and the configuration do not have does not exist
+    less = {n: st.f32(n) for n in st.names() if not n.endswith((".b", "dwa", "shared.sg"))}
+    cfg2 = json.loads(json.dumps(ZCFG))
+    del cfg2["layers"][0]["mixer"]["softcap"], cfg2["layers"][0]["mixer"]["q_temp"], cfg2["norm"]["groups"]
+    synth.write_seq_model_dir(str(tmp_path / "less"), cfg2, 1, tensors=less)
+    layers, top = seqmodel.ARCHITECTURES["Zusolix"](cfg2, safetensors_io.SafeTensors(str(tmp_path / "less" / "model.safetensors")), FakeUp())
+    a, g, _ = layers
+    assert (a.in_bias, g.in_bias, a.depth_mix, a.shared_gate, a.softcap, a.qtemp_every, top["norm_groups"]) == (None, None, None, None, 0.0, 0, 1) and a.shared_up is not None
+    for key, val in (("type", "conveyor"), ("mlp", {"kind": "sparse", "ff": 8})):
+        bad = json.loads(json.dumps(ZCFG))
+        bad["layers"][1][key] = val
+        with pytest.raises(seqmodel.ConfigError):
+            seqmodel.ARCHITECTURES["Zusolix"](bad, st, FakeUp())
+    bad = json.loads(json.dumps(ZCFG))
+    bad["layers"][0]["mlp"]["router"]["top"] = 4
+    with pytest.raises(seqmodel.ConfigError):
+        seqmodel.ARCHITECTURES["Zusolix"](bad, st, FakeUp())
+
+
+def test_plain_zusolix_statement_reach_and_pieces():
+    """causal, and every later token sees a changed one (nothing limits the reach); the norm's groups are on their own; the temperature steps where it should;
+    the largest scores are the ones chosen"""
+    t = synth.seq_tensors(ZCFG, 2)
+    rng = np.random.default_rng(0)
+    a = rng.integers(0, 30, 20)
+    b = a.copy()
+    b[6] = (b[6] + 1) % 30
+    la, lb = seq_oracle.run_zusolix(ZCFG, t, a), seq_oracle.run_zusolix(ZCFG, t, b)
+    assert np.array_equal(la[:6], lb[:6]) and min(np.abs(la[i] - lb[i]).max() for i in range(6, 20)) > 1e-6
+    x = rng.standard_normal((4, 12))
+    y = x.copy()
+    y[:, 4:8] *= 7.0  # scaling one part changes nothing (up to eps), inside or outside it
+    assert np.abs(seq_oracle.grouped_norm(x, np.ones(12), 3, 0.0) - seq_oracle.grouped_norm(y, np.ones(12), 3, 0.0)).max() < 1e-12
+    assert np.abs(seq_oracle.grouped_norm(x, np.ones(12), 1, 0.0) - seq_oracle.grouped_norm(y, np.ones(12), 1, 0.0)).max() > 0.1
+    assert [round(float(seq_oracle.query_temperature(p, 1.0, 4)), 6) for p in (0, 2, 3, 6, 7)] == [1.0, 1.0, round(1 + np.log(2), 6), round(1 + np.log(2), 6), round(1 + np.log(3), 6)]
+    W = {k: np.asarray(v, np.float64) for k, v in t.items()}
+    h = rng.standard_normal((5, 24))
+    mlp = ZCFG["layers"][0]["mlp"]
+    full = seq_oracle.expert_mixture(W, "l0.mlp.", h, mlp, use_shared=False)
+    for i in range(5):
+        s = seq_oracle.sigmoid(W["l0.mlp.router"] @ h[i])
+        keep = np.argsort(-s)[:2]
+        assert np.allclose(full[i], sum(seq_oracle.one_expert(W, "l0.mlp.e%d." % e, s[e] * h[i]) for e in keep))
 
 
 def test_the_small_library_exports_what_its_models_need():
