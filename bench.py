@@ -54,7 +54,9 @@ def parse():
     ap.add_argument("--f16-super-chunk", type=int, default=2048, help="side leg (fp16 perf mode): tokens per mat-mul launch")
     ap.add_argument("--layer-list", default=None, metavar="SIZES", help="instead of the headline workload: prefill / decode throughput of a layer-list model (dense bf16 "
                     "matrices; powerserve_amd/bench_seq.py SIZES, comma-separated, or 'all'): the sizes 2048x6 / 4096x3 beside the Q4_K Llama path at equal width, "
-                    "the sizes v2048x6 / v4096x3 (parallel layers, windowed attention with pooled blocks beside gated linear attention) beside the layer-list model of equal size")
+                    "the sizes v2048x6 / v4096x3 (parallel layers, windowed attention with pooled blocks beside gated linear attention) beside the layer-list model of equal size, "
+                    "the sizes z2048x6 / z4096x3 (Zusolix: depth-averaged parallel layers, soft-capped causal attention or a gated recurrence, mixture-of-experts feed-forwards) "
+                    "beside the v sizes")
     ap.add_argument("--layer-list-portion", type=int, default=512, help="--layer-list: tokens per launch sequence of the prefill")
     ap.add_argument("--prefill-warmup-tokens", type=int, default=128, help="untimed tokens forwarded before the timed prefill (first use of the prefill kernels in the process; 0: none)")
     ap.add_argument("--wide-chunk", type=int, default=512, help="side leg: prefill in chunks of this many tokens (0: skip)")

@@ -23,11 +23,24 @@ SIZES = {
                     layers=4, loop=(1, 3, 2), beside="2048x6"),
     "v4096x3": dict(design="Vobisun", width=4096, ff=14336, heads=32, kv_heads=8, dim=128, window=1024, pool=64, rot_dims=64, lin_heads=32, lin_dim=64, lin_vdim=128,
                     layers=3, loop=None, beside="4096x3"),
+    # Zusolix (two-norm parallel layers with a depth average; causal attention with a soft cap and a query temperature, or an element-wise gated recurrence;
+    # the first layer's feed-forward dense, the others 8 experts of which a token uses 2, plus a shared one: 2 x ff/4 + ff/2 = ff active rows) beside the
+    # Vobisun model of equal width, feed-forward size, head counts and layer runs
+    "z2048x6": dict(design="Zusolix", width=2048, ff=8192, heads=16, kv_heads=4, dim=128, gru=3072, experts=8, top=2, order="aagaag", layers=6, beside="v2048x6"),
+    "z4096x3": dict(design="Zusolix", width=4096, ff=14336, heads=32, kv_heads=8, dim=128, gru=6144, experts=8, top=2, order="aga", layers=3, beside="v4096x3"),
 }
 
 
 def config(z: dict, vocab: int = 4096) -> dict:
     H, d = z["heads"], z["dim"]
+    if z.get("design") == "Zusolix":
+        att = synth.zusolix_attention(H, z["kv_heads"], d, d, float(d ** -0.5), 30.0, (0.1, 1024))
+        layers = []
+        for i, k in enumerate(z["order"]):
+            mixer = ("attention", att) if k == "a" else ("mingru", {"width": z["gru"]})
+            layers.append(synth.zusolix_layer(*mixer, ff=z["ff"]) if i == 0 else
+                          synth.zusolix_layer(*mixer, moe=(z["experts"], z["top"], z["ff"] // 4), shared=z["ff"] // 2))
+        return synth.zusolix_config(z["width"], vocab, layers, groups=4, embed_scale=float(z["width"] ** 0.5), residual_mult=0.5)
     if z.get("design") == "Vobisun":
         left = dict(heads=H, kv_heads=z["kv_heads"], dim=d, vdim=d, mask={"size": z["window"], "pool": z["pool"]},
                     rot={"base": 1e6, "dims": z["rot_dims"], "scaling": {"factor": 4.0}}, scale=float(d ** -0.5))
@@ -59,7 +72,7 @@ def _kernel(ctx, m, which, T, reps):
     return us.value, by.value, fl.value
 
 
-def run_size(ctx, name: str, prompt_len: int, steps: int, max_batch: int, seed: int = 0, with_llama: bool = True) -> dict:
+def run_size(ctx, name: str, prompt_len: int, steps: int, max_batch: int, seed: int = 0, with_llama: bool = True, with_beside: bool = True) -> dict:
     z = SIZES[name]
     cfg = config(z)
     out = {"size": name, "config": {k: v for k, v in z.items() if k not in ("llama", "beside")}, "prompt_len": prompt_len, "decode_steps": steps, "portion": max_batch}
@@ -88,9 +101,15 @@ def run_size(ctx, name: str, prompt_len: int, steps: int, max_batch: int, seed: 
     out["ff_up_matvec"] = {"us": us, "GBs": by / us / 1e3, "hbm_frac": by / us / 1e3 / HBM_PEAK_GBS}
     us, by, fl = _kernel(ctx, m, 0, max_batch, 5)
     out["ff_up_matmul"] = {"tokens": max_batch, "us": us, "TFLOPs": fl / us / 1e6, "mfma_frac": fl / us / 1e6 / MFMA_BF16_PEAK_TFLOPS}
+    if z.get("experts"):  # the experts' grouped products: up (gate / up rows, SiLU pair) and down, a single token and a portion
+        for which, key in ((2, "moe_up"), (3, "moe_down")):
+            us, by, fl = _kernel(ctx, m, which, 1, 20)
+            out[key + "_matvec"] = {"us": us, "GBs": by / us / 1e3, "hbm_frac": by / us / 1e3 / HBM_PEAK_GBS}
+            us, by, fl = _kernel(ctx, m, which, max_batch, 5)
+            out[key + "_matmul"] = {"tokens": max_batch, "us": us, "TFLOPs": fl / us / 1e6, "mfma_frac": fl / us / 1e6 / MFMA_BF16_PEAK_TFLOPS}
     m.close()
-    if z.get("beside"):  # the closest existing model at equal size, same workload
-        out["beside"] = run_size(ctx, z["beside"], prompt_len, steps, max_batch, seed, with_llama=False)
+    if with_beside and z.get("beside"):  # the closest existing model at equal size, same workload
+        out["beside"] = run_size(ctx, z["beside"], prompt_len, steps, max_batch, seed, with_llama=False, with_beside=False)
     if with_llama and z.get("llama"):
         with tempfile.TemporaryDirectory() as d:
             synth.write_model_dir(d, z["llama"], gguf.Q4_K, n_ctx=prompt_len + steps + 64, seed=seed)

@@ -292,8 +292,9 @@ __global__ __launch_bounds__(256) void dense_mv_kernel(dn_args g) {
 
 
 // Grouped mat-vec (ps_seq.h, grouped products): block row r = one output row, which adds its g_inner slots; slot s = r g_inner + i reads A row s / g_adiv
-// times g_scale[s] and the matrix g_sel[s].  Dynamic LDS: [g_inner][Kp] activations, rounded as in dense_mv_kernel.  The same four-rows-per-wave walk.
-template <typename WT>
+// times g_scale[s] and the matrix g_sel[s].  Dynamic LDS: [g_inner][Kp] activations, rounded as in dense_mv_kernel.  A wave streams RW weight rows at a
+// time, two 16-byte pieces of each in flight; small matrices take fewer rows per wave so that the launch still has waves for every CU.
+template <typename WT, int RW>
 __global__ __launch_bounds__(256) void dense_mv_grouped_kernel(dn_args g) {
     extern __shared__ __attribute__((aligned(16))) float xs[]; // [inner][Kp]
     const long long K = g.K, Kp = (K + 7) / 8 * 8;
@@ -307,7 +308,7 @@ __global__ __launch_bounds__(256) void dense_mv_grouped_kernel(dn_args g) {
     }
     __syncthreads();
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    constexpr int RW = 4, VE = 16 / (int)sizeof(WT);
+    constexpr int VE = 16 / (int)sizeof(WT);
     const bool vec = (K * (long long)sizeof(WT)) % 16 == 0;
     for (long long nb = ((long long)blockIdx.x * 4 + wave) * RW; nb < g.N; nb += (long long)gridDim.x * 4 * RW) {
         float acc[RW];
@@ -317,26 +318,33 @@ __global__ __launch_bounds__(256) void dense_mv_grouped_kernel(dn_args g) {
             const WT *W = (const WT *)g.w + (long long)g.g_sel[(long long)r * inner + c] * g.wstride;
             const float *x = xs + (long long)c * Kp;
             if (vec) {
-                for (long long k = (long long)lane * VE; k < K; k += 64 * VE) {
-                    dn_f4 raw[RW];
+                for (long long k = (long long)lane * VE; k < K; k += 128 * VE) {
+                    const long long k2 = k + 64 * VE;
+                    const bool two = k2 < K;
+                    dn_f4 raw[2][RW];
 #pragma unroll
                     for (int q = 0; q < RW; q++) {
                         const long long n = nb + q < g.N ? nb + q : g.N - 1;
-                        raw[q] = __builtin_nontemporal_load((const dn_f4 *)(W + n * K + k));
+                        raw[0][q] = __builtin_nontemporal_load((const dn_f4 *)(W + n * K + k));
+                        raw[1][q] = two ? __builtin_nontemporal_load((const dn_f4 *)(W + n * K + k2)) : dn_f4{0.f, 0.f, 0.f, 0.f};
                     }
 #pragma unroll
-                    for (int q = 0; q < RW; q++) {
-                        float wv[VE];
-                        if constexpr (sizeof(WT) == 2) {
-                            unsigned short h[8];
-                            __builtin_memcpy(h, &raw[q], 16);
+                    for (int u = 0; u < 2; u++) {
+                        const long long ku = u ? (two ? k2 : k) : k; // (the second piece is zero where there is none: any valid x offset will do)
 #pragma unroll
-                            for (int e = 0; e < 8; e++) wv[e] = dn_bf2f(h[e]);
-                        } else {
-                            __builtin_memcpy(wv, &raw[q], 16);
+                        for (int q = 0; q < RW; q++) {
+                            float wv[VE];
+                            if constexpr (sizeof(WT) == 2) {
+                                unsigned short h[8];
+                                __builtin_memcpy(h, &raw[u][q], 16);
+#pragma unroll
+                                for (int e = 0; e < 8; e++) wv[e] = dn_bf2f(h[e]);
+                            } else {
+                                __builtin_memcpy(wv, &raw[u][q], 16);
+                            }
+#pragma unroll
+                            for (int e = 0; e < VE; e++) acc[q] = fmaf(wv[e], x[ku + e], acc[q]);
                         }
-#pragma unroll
-                        for (int e = 0; e < VE; e++) acc[q] = fmaf(wv[e], x[k + e], acc[q]);
                     }
                 }
             } else {
@@ -357,8 +365,16 @@ __global__ __launch_bounds__(256) void dense_mv_grouped_kernel(dn_args g) {
             for (int o = 32; o > 0; o >>= 1) acc[q] += __shfl_xor(acc[q], o, 64);
         }
 #pragma unroll
-        for (int q = 0; q < RW; q++) dn_put(g, r, nb + q, acc[q], acc[q ^ 1], lane == 0 && nb + q < g.N);
+        for (int q = 0; q < RW; q++) dn_put(g, r, nb + q, acc[q], acc[RW > 1 ? (q ^ 1) : q], lane == 0 && nb + q < g.N);
     }
+}
+template <typename WT, int RW>
+static void dn_launch_mv_grouped(hipStream_t st, const dn_args &g, int rows, size_t lds) {
+    static unsigned long long mask = 0;
+    if (ps_first_on_device(&mask)) (void)hipFuncSetAttribute((const void *)dense_mv_grouped_kernel<WT, RW>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    long long blocks = (g.N + 4 * RW - 1) / (4 * RW);
+    if (blocks > 2048) blocks = 2048;
+    hipLaunchKernelGGL((dense_mv_grouped_kernel<WT, RW>), dim3((unsigned)blocks, (unsigned)rows), dim3(256), lds, st, g);
 }
 
 // ---------------------------------------------------------------------------------------------------- wide mat-mul (bf16, K % 64 == 0)
@@ -475,17 +491,19 @@ int psk_dense(hipStream_t st, const psk_dense_args &a) {
     if (a.groups > 0) {
         g.groups = a.groups; g.N = a.w->N / a.groups; g.wstride = g.N * g.K;
         g.g_adiv = a.g_adiv; g.g_odiv = a.g_odiv; g.g_inner = a.g_inner; g.g_sel = a.g_sel; g.g_scale = a.g_scale;
-        if (!a.g_list) { // a mat-vec per output row (T rows of g_inner slots each)
-            static unsigned long long mask = 0;
-            if (ps_first_on_device(&mask)) {
-                (void)hipFuncSetAttribute((const void *)dense_mv_grouped_kernel<unsigned short>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-                (void)hipFuncSetAttribute((const void *)dense_mv_grouped_kernel<float>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (!a.g_list) { // a mat-vec per output row (T rows of g_inner slots each); four rows per wave only where that still leaves about 1024 waves
+            const long long waves4 = (g.N + 3) / 4 * a.T;
+            const int RW = waves4 >= 1024 ? 4 : (waves4 >= 512 || g.act == PSD_ACT_SILU_PAIR) ? 2 : 1; // (a gate / up pair sits in one wave)
+            const size_t lds = kp4 * a.g_inner;
+            if (bf) {
+                if (RW == 4) dn_launch_mv_grouped<unsigned short, 4>(st, g, a.T, lds);
+                else if (RW == 2) dn_launch_mv_grouped<unsigned short, 2>(st, g, a.T, lds);
+                else dn_launch_mv_grouped<unsigned short, 1>(st, g, a.T, lds);
+            } else {
+                if (RW == 4) dn_launch_mv_grouped<float, 4>(st, g, a.T, lds);
+                else if (RW == 2) dn_launch_mv_grouped<float, 2>(st, g, a.T, lds);
+                else dn_launch_mv_grouped<float, 1>(st, g, a.T, lds);
             }
-            long long blocks = (g.N + 15) / 16;
-            if (blocks > 2048) blocks = 2048;
-            const dim3 grid((unsigned)blocks, (unsigned)a.T);
-            if (bf) hipLaunchKernelGGL(dense_mv_grouped_kernel<unsigned short>, grid, dim3(256), kp4 * a.g_inner, st, g);
-            else hipLaunchKernelGGL(dense_mv_grouped_kernel<float>, grid, dim3(256), kp4 * a.g_inner, st, g);
             return 0;
         }
         g.g_seg = a.g_seg; g.g_list = a.g_list;

@@ -44,13 +44,13 @@ void psk_rmsnorm(hipStream_t st, const float *x, int64_t ldx, const int32_t *idx
 // of them as it is), kept in xout (NULL: not kept; it may be the last stream itself); then, over `groups` equal parts of the row each with its own mean square,
 // h = x / rms * (offset + w1) and h2 = x / rms * (offset + w2): two norms of the same vector share their statistics (w1 / w2 NULL: not wanted).
 // dynamic LDS: n + groups floats.
-__global__ __launch_bounds__(256) void sq_front_kernel(const float *src, long long stride, int nmix, const float *mix, const int32_t *idx, float *xout, const float *w1,
+__global__ __launch_bounds__(1024) void sq_front_kernel(const float *src, long long stride, int nmix, const float *mix, const int32_t *idx, float *xout, const float *w1,
                                                        float *h, const float *w2, float *h2, int groups, float offset, float eps, long long n) {
     extern __shared__ float fr[];
     float *xs = fr, *inv = fr + n;
     const long long r = idx ? idx[blockIdx.x] : blockIdx.x, o = (long long)blockIdx.x * n;
-    const int tid = threadIdx.x;
-    for (long long i = tid; i < n; i += 256) {
+    const int tid = threadIdx.x, nt = blockDim.x;
+    for (long long i = tid; i < n; i += nt) {
         float v;
         if (mix) {
             v = 0.f;
@@ -64,7 +64,7 @@ __global__ __launch_bounds__(256) void sq_front_kernel(const float *src, long lo
     if (!w1 && !w2) return;
     __syncthreads();
     const long long gs = n / groups;
-    for (int g = tid >> 6; g < groups; g += 4) {
+    for (int g = tid >> 6; g < groups; g += nt >> 6) {
         float s = 0.f;
         for (long long i = tid & 63; i < gs; i += 64) s += xs[g * gs + i] * xs[g * gs + i];
 #pragma unroll
@@ -72,7 +72,7 @@ __global__ __launch_bounds__(256) void sq_front_kernel(const float *src, long lo
         if ((tid & 63) == 0) inv[g] = 1.f / sqrtf(s / (float)gs + eps);
     }
     __syncthreads();
-    for (long long i = tid; i < n; i += 256) {
+    for (long long i = tid; i < n; i += nt) {
         const float v = xs[i] * inv[i / gs];
         if (w1) h[o + i] = v * (offset + w1[i]);
         if (w2) h2[o + i] = v * (offset + w2[i]);
@@ -83,7 +83,7 @@ void psk_front(hipStream_t st, const float *src, int64_t stride, int nmix, const
     if (rows <= 0) return;
     static unsigned long long mask = 0;
     if (ps_first_on_device(&mask)) (void)hipFuncSetAttribute((const void *)sq_front_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    hipLaunchKernelGGL(sq_front_kernel, dim3(rows), dim3(256), (size_t)(n + groups) * 4, st, src, (long long)stride, nmix, mix, idx, xout, w1, h, w2, h2, groups, offset, eps,
+    hipLaunchKernelGGL(sq_front_kernel, dim3(rows), dim3(rows <= 8 && n >= 2048 ? 1024 : 256), (size_t)(n + groups) * 4, st, src, (long long)stride, nmix, mix, idx, xout, w1, h, w2, h2, groups, offset, eps,
                        (long long)n);
 }
 

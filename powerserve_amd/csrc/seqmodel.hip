@@ -751,14 +751,44 @@ int ps_hip_seq_decode_greedy(ps_hip_seq *m, int slot, int32_t token, int steps, 
 
 int ps_hip_seq_bench_kernel(ps_hip_seq *m, int which, int T, int reps, double *us, double *bytes, double *flops) {
     ps_hip_ctx *c = m->ctx;
-    if (T <= 0 || T > m->d.max_batch || reps <= 0 || which < 0 || which > 1) return seq_fail(c, "seq_bench_kernel: bad argument");
+    if (T <= 0 || T > m->d.max_batch || reps <= 0 || which < 0 || which > 3) return seq_fail(c, "seq_bench_kernel: bad argument");
     PS_CHECK(c, hipSetDevice(c->device));
+    const bool moe = which >= 2;
+    const int64_t W = m->d.width;
+    if (moe) { // tokens 0, 1, 2, ... embedded as the input: a routing as spread as the router's rows make it
+        std::vector<int32_t> ids((size_t)T);
+        for (int i = 0; i < T; i++) ids[i] = i % m->d.vocab;
+        PS_CHECK(c, hipMemcpyAsync(m->tokens, ids.data(), (size_t)T * 4, hipMemcpyHostToDevice, c->stream));
+        psk_embed(c->stream, m->d.embed, m->tokens, m->step, T, m->embed_scale, m->h, W);
+        PS_CHECK(c, hipStreamSynchronize(c->stream));
+    } else {
+        psk_fill(c->stream, m->h, 0.01f, (int64_t)m->d.max_batch * W);
+    }
     std::vector<psk_dense_args> launches; // one per layer that has the matrix: every launch streams its own (cold) weights, as in a step
+    double per_bytes = 0, per_flops = 0;
     for (const LayerPlan &P : m->L) {
-        if (P.d.ff_kind == PS_FF_NONE) continue;
+        if (P.d.ff_kind == PS_FF_NONE || (P.d.ff_kind == PS_FF_MOE_SWIGLU) != moe) continue;
         psk_dense_args g;
         g.T = T; g.pack = m->pack; g.pack_bytes = m->pack_bytes;
-        if (which == 0) {
+        if (moe) {
+            // the routing of this layer (all layers' launches below then reuse the LAST layer's routing: the same shapes and spread)
+            const int top = P.d.top, S = T * top;
+            const bool mv = T <= 8;
+            psk_moe_route(c->stream, m->h, W, P.d.router, P.d.shared_gate, P.d.experts, top, P.d.moe_norm_top, W, T, m->moe_sel, m->moe_wgt, m->moe_sg);
+            if (!mv) psk_moe_plan(c->stream, m->moe_sel, S, P.d.experts, m->moe_seg, m->moe_list);
+            g.groups = P.d.experts; g.g_sel = m->moe_sel;
+            if (!mv) { g.g_seg = m->moe_seg; g.g_list = m->moe_list; }
+            if (which == 2) {
+                g.w = P.d.ff_up; g.a = m->h; g.lda = W; g.out = m->t4; g.ldo = P.d.ff; g.act = PSD_ACT_SILU_PAIR; g.T = S; g.g_adiv = top; g.g_scale = m->moe_wgt;
+            } else {
+                g.w = P.d.ff_down; g.a = m->t4; g.lda = P.d.ff; g.ldo = W;
+                if (mv) { g.T = T; g.g_inner = top; g.out = m->y; }
+                else { g.T = S; g.out = top == 1 ? m->y : m->moe_y; }
+            }
+            const int used = std::min(P.d.experts, S); // matrices a launch can touch at most
+            per_bytes = (double)dense_bytes(g.w) / P.d.experts * used;
+            per_flops = 2.0 * S * (double)(g.w->N / P.d.experts) * (double)g.w->K;
+        } else if (which == 0) {
             g.w = P.d.ff_up; g.a = m->h; g.lda = m->d.width; g.out = m->t4; g.ldo = P.d.ff;
             if (P.d.ff_kind == PS_FF_DENSE_SWIGLU) g.act = PSD_ACT_SILU_PAIR;
             else { g.act = PSD_ACT_XIELU; g.act_p = P.act_p; g.act_q = P.act_q; }
@@ -767,7 +797,6 @@ int ps_hip_seq_bench_kernel(ps_hip_seq *m, int which, int T, int reps, double *u
         launches.push_back(g);
     }
     if (launches.empty()) return seq_fail(c, "seq_bench_kernel: no layer has a feed-forward");
-    psk_fill(c->stream, m->h, 0.01f, (int64_t)m->d.max_batch * m->d.width);
     hipEvent_t e0, e1;
     PS_CHECK(c, hipEventCreate(&e0));
     PS_CHECK(c, hipEventCreate(&e1));
@@ -782,8 +811,8 @@ int ps_hip_seq_bench_kernel(ps_hip_seq *m, int which, int T, int reps, double *u
     (void)hipEventDestroy(e0);
     (void)hipEventDestroy(e1);
     *us = 1e3 * ms / ((double)reps * launches.size());
-    *bytes = (double)dense_bytes(launches[0].w);
-    *flops = 2.0 * T * (double)launches[0].w->N * (double)launches[0].w->K;
+    *bytes = moe ? per_bytes : (double)dense_bytes(launches[0].w);
+    *flops = moe ? per_flops : 2.0 * T * (double)launches[0].w->N * (double)launches[0].w->K;
     return 0;
 }
 
