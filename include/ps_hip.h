@@ -318,11 +318,14 @@ enum ps_ff_kind {
     PS_FF_DENSE_XIELU = 1,  /* W_down xIELU(W_up h) */
     PS_FF_DENSE_SWIGLU = 2, /* W_down (silu(W_gate h) * (W_up h)); ff_up holds the rows of gate and up INTERLEAVED (gate_0, up_0, gate_1, ...): [2 ff, width] */
     PS_FF_MOE_SWIGLU = 3,   /* `experts` feed-forwards of the SWIGLU form of which a token uses `top` (fields below), plus an optional shared one */
+    PS_FF_DENSE_RELU_GLU = 4, /* W_down (relu(W_gate h + b) * (W_up h + b)) + b; ff_up interleaved as for SWIGLU, ff_up_bias [2 ff] interleaved alike, ff_down_bias [width] (either NULL: none) */
+    PS_FF_MOE_RELU2 = 5,    /* a mixture of experts of the form W_down relu(W_up h)^2: ff_up [experts * ff, width], ff_down [experts * width, ff], shared_up [shared_ff, width] */
 };
 enum ps_layer_form {
     PS_LAYER_SEQUENTIAL = 0, /* x += norm_b(mixer(conv(norm1(x)))), then x += norm_b(ff(conv(norm2(x)))) */
     PS_LAYER_PARALLEL   = 1, /* h = norm1(x); x += res_scale (mixer(conv(h)) + ff(h2)): no norm behind the sublayers, only the mixer's input is filtered (canon1 NULL:
                               * not at all); h2 = h, or norm2(x) where norm2 is given (two weights over the same statistics) */
+    PS_LAYER_PRENORM    = 2, /* x += mixer(norm1(x)), then x += ff(norm2(x)): the second norm reads what the mixer left; no input filter, nothing normed behind a sublayer */
 };
 enum ps_rot_pairing { PS_ROT_HALVES = 0 /* (i, i + dims/2) */, PS_ROT_NEIGHBOURS = 1 /* (2i, 2i + 1) */ };
 
@@ -393,6 +396,25 @@ typedef struct ps_seq_layer_s {
     int32_t experts, top, shared_ff, moe_norm_top;
     const float *router, *shared_gate;
     const ps_dense *shared_up, *shared_down;
+    /* ---- attention extras (PS_MIX_WINATTN), continued */
+    int32_t head_norm;                  /* 1: qnorm / knorm are [dim] weights of RMS norms taken per HEAD (one weight vector shared by the heads) instead of over the whole projection */
+    int32_t v_unit;                     /* 1: every head's value is divided by its own root mean square (eps inside the root, no weight) before it is cached */
+    /* gated == 2 (PS_MIX_WINATTN): the gate projection has heads * vdim rows and multiplies the concatenated heads element by element.
+     * PS_MIX_LATENT reads gated too (1: a row per head; in_cat then ends with the gate's rows), and with q_rank == 0 its queries come straight from the input:
+     *   in_cat = rows of q | dkv | gate ([heads * (dim + rot_dim) + kv_rank + rot_dim + (gated ? heads : 0), width]), uq and qnorm unused; window 0 = everything before the token */
+    /* ---- rotary frequency scaling by wavelength (PS_MIX_LATENT; yarn_factor 0: none): with dim(t) = rot_dims ln(yarn_original / (2 pi t)) / (2 ln rot_base),
+     * lo = max(floor(dim(yarn_fast)), 0), hi = min(ceil(dim(yarn_slow)), rot_dims - 1), ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1), pair i turns with
+     * f_i / yarn_factor * ramp_i + f_i (1 - ramp_i), and cos and sin are both multiplied by 0.1 ln(yarn_factor) + 1 */
+    float yarn_factor, yarn_fast, yarn_slow;
+    int32_t yarn_original;
+    /* ---- feed-forward extras */
+    const float *ff_up_bias, *ff_down_bias; /* PS_FF_DENSE_RELU_GLU / PS_FF_DENSE_SWIGLU: biases of the (interleaved) gate / up rows and of the down rows, or NULL */
+    /* mixtures of experts: `experts` counts the feed-forwards that have tensors; the router has experts + moe_identity rows, the last moe_identity of which are
+     * identity experts (their output is their input).  moe_softmax 1: scores = soft-max over all router rows (0: sigmoid).  moe_correction [router rows] or NULL is added
+     * to the scores for the CHOICE only.  moe_groups > 0: the router rows form that many equal groups of neighbours, a group's score is its largest choice score, and
+     * only rows of the moe_keep best groups can be chosen.  moe_weight_output 1: a chosen expert's score multiplies its output (0: its input). */
+    int32_t moe_identity, moe_softmax, moe_groups, moe_keep, moe_weight_output;
+    const float *moe_correction;
 } ps_seq_layer;
 
 typedef struct {
@@ -410,6 +432,7 @@ typedef struct {
     int32_t loop_start, loop_stop, loop_times;
     int32_t max_context; /* most tokens a sequence may hold: sizes what grows with a sequence (the pooled blocks of PS_MIX_WINATTN, a window of everything); 0: 65536 */
     int32_t norm_groups; /* every RMS norm over the width is taken in this many equal consecutive parts, each with its own mean square (0 is taken as 1) */
+    int32_t norm_center; /* 1: the norms over the width are layer norms -- the mean is taken off first and the variance is the mean of the squared deviations (PS_LAYER_PRENORM layers and the final norm) */
 } ps_seq_desc;
 
 int ps_hip_seq_create(ps_hip_ctx *ctx, const ps_seq_desc *desc, ps_hip_seq **out);

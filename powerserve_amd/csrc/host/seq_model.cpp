@@ -410,10 +410,158 @@ void zusolix(const JsonValue &cfg, const SafeTensorsFile &st, SeqUploader &up, s
         layers.push_back(L);
     }
 }
+// ---------------------------------------------------------------- Pokatar: pre-norm layers with layer norms, sink attention / shared-key latent attention, relu-gated dense / squared-relu expert feed-forwards
+void check_rows(const SafeTensorsFile &st, const std::string &n, int64_t rows) {
+    if (rows_of(st, n) != rows) POWERSERVE_ABORT("tensor " + n + ": its rows are not what the configuration gives");
+}
+void sink_attention_mixer(ps_seq_layer &L, const SafeTensorsFile &st, SeqUploader &up, const std::string &m, const JsonValue &mc) {
+    L.kind = PS_MIX_WINATTN;
+    L.heads = (int32_t)mc.at("heads").num;
+    L.dim = (int32_t)mc.at("dim").num;
+    L.kv_heads = (int32_t)num_or(mc, "kv_heads", L.heads);
+    L.vdim = (int32_t)num_or(mc, "vdim", L.dim);
+    if (L.kv_heads <= 0 || L.heads % L.kv_heads) POWERSERVE_ABORT(m + ": heads over key / value heads");
+    if (const JsonValue *mask = obj_or_null(mc, "mask")) L.window = (int32_t)num_or(*mask, "size", 0);
+    L.rot_pairing = PS_ROT_HALVES;
+    L.rot_base = 10000.f;
+    L.scale = (float)num_or(mc, "scale", 1.0 / std::sqrt((double)L.dim));
+    L.head_norm = 1; // q / k norms per head, one weight vector of `dim`
+    L.v_unit = 1;    // every head's value a unit-rms vector
+    std::vector<std::string> names = {m + "q", m + "k", m + "v"};
+    check_rows(st, m + "q", (int64_t)L.heads * L.dim);
+    check_rows(st, m + "k", (int64_t)L.kv_heads * L.dim);
+    check_rows(st, m + "v", (int64_t)L.kv_heads * L.vdim);
+    if (st.contains(m + "g")) {
+        check_rows(st, m + "g", (int64_t)L.heads * L.vdim);
+        L.gated = 2; // a gate row per output element
+        names.push_back(m + "g");
+    }
+    L.in_cat = mat_rows(st, up, names);
+    if (st.contains(m + "q.norm")) L.qnorm = up.vec(expect1(st, m + "q.norm", L.dim));
+    if (st.contains(m + "k.norm")) L.knorm = up.vec(expect1(st, m + "k.norm", L.dim));
+    L.sink = up.vec(std::vector<float>((size_t)L.heads, 0.f)); // exp(0) = 1 joins every head's denominator
+    L.out = mat1(st, up, m + "o");
+}
+void shared_key_latent_mixer(ps_seq_layer &L, const SafeTensorsFile &st, SeqUploader &up, const std::string &m, const JsonValue &mc) {
+    L.kind = PS_MIX_LATENT;
+    L.q_rank = 0; // the queries come straight from the input
+    L.heads = (int32_t)mc.at("heads").num;
+    L.dim = (int32_t)mc.at("dim").num;
+    L.vdim = (int32_t)num_or(mc, "vdim", L.dim);
+    L.kv_rank = (int32_t)mc.at("kv_rank").num;
+    L.rot_dim = (int32_t)mc.at("rot_dim").num;
+    L.rot_base = 10000.f;
+    if (const JsonValue *rot = obj_or_null(mc, "rot")) {
+        L.rot_dims = (int32_t)num_or(*rot, "dims", 0);
+        L.rot_base = (float)num_or(*rot, "base", 10000.0);
+        if (const JsonValue *sc = obj_or_null(*rot, "scaling")) {
+            L.yarn_factor = (float)sc->at("factor").num;
+            L.yarn_fast = (float)sc->at("fast").num;
+            L.yarn_slow = (float)sc->at("slow").num;
+            L.yarn_original = (int32_t)sc->at("original").num;
+        }
+    }
+    if (const JsonValue *mask = obj_or_null(mc, "mask")) L.window = (int32_t)num_or(*mask, "size", 0);
+    L.scale = (float)mc.at("scale").num;
+    std::vector<std::string> names = {m + "q", m + "dkv"};
+    check_rows(st, m + "q", (int64_t)L.heads * (L.dim + L.rot_dim));
+    check_rows(st, m + "dkv", (int64_t)L.kv_rank + L.rot_dim);
+    check_rows(st, m + "uk", (int64_t)L.heads * L.dim);
+    check_rows(st, m + "uv", (int64_t)L.heads * L.vdim);
+    if (st.contains(m + "g")) {
+        check_rows(st, m + "g", L.heads);
+        L.gated = 1;
+        names.push_back(m + "g");
+    }
+    L.in_cat = mat_rows(st, up, names);
+    L.ukv = mat_rows(st, up, {m + "uk", m + "uv"});
+    L.kvnorm = up.vec(expect1(st, m + "dkv.norm", L.kv_rank));
+    L.out = mat1(st, up, m + "o");
+}
+void relu_feed_forward(ps_seq_layer &L, const SafeTensorsFile &st, SeqUploader &up, const std::string &p, const JsonValue &f, int64_t W) {
+    const std::string kind = f.at("kind").str;
+    if (kind == "dense") {
+        L.ff_kind = PS_FF_DENSE_RELU_GLU;
+        L.ff = (int32_t)f.at("ff").num;
+        std::vector<uint16_t> both;
+        append_gate_up(st, p, L.ff, W, both);
+        L.ff_up = up.mat(both, 2 * (int64_t)L.ff, W);
+        L.ff_down = mat1(st, up, p + "down");
+        if (st.contains(p + "gate.b") || st.contains(p + "up.b")) {
+            const std::vector<float> zero((size_t)L.ff, 0.f);
+            const auto g = st.contains(p + "gate.b") ? expect1(st, p + "gate.b", L.ff) : zero, u = st.contains(p + "up.b") ? expect1(st, p + "up.b", L.ff) : zero;
+            std::vector<float> b(2 * (size_t)L.ff);
+            for (int64_t r = 0; r < L.ff; r++) { b[2 * r] = g[r]; b[2 * r + 1] = u[r]; }
+            L.ff_up_bias = up.vec(b);
+        }
+        if (st.contains(p + "down.b")) L.ff_down_bias = up.vec(expect1(st, p + "down.b", W));
+    } else if (kind == "moe") {
+        const JsonValue &r = f.at("router");
+        L.ff_kind = PS_FF_MOE_RELU2;
+        L.ff = (int32_t)f.at("expert").at("ff").num;
+        L.experts = (int32_t)r.at("experts").num;
+        L.top = (int32_t)r.at("top").num;
+        L.moe_identity = (int32_t)num_or(r, "identity", 0);
+        L.moe_softmax = 1;
+        L.moe_weight_output = 1;
+        if (const JsonValue *gr = obj_or_null(r, "groups")) { L.moe_groups = (int32_t)num_or(*gr, "count", 0); L.moe_keep = (int32_t)num_or(*gr, "keep", 0); }
+        const int rows = L.experts + L.moe_identity;
+        if (L.experts <= 0 || L.top <= 0 || L.top > rows) POWERSERVE_ABORT(p + ": top / experts");
+        std::vector<std::string> ups, downs;
+        for (int e = 0; e < L.experts; e++) {
+            const std::string pe = p + "e" + std::to_string(e) + ".";
+            if (rows_of(st, pe + "up") != L.ff || cols_of(st, pe + "up") != W || rows_of(st, pe + "down") != W || cols_of(st, pe + "down") != L.ff) POWERSERVE_ABORT(pe + ": expert shapes");
+            ups.push_back(pe + "up");
+            downs.push_back(pe + "down");
+        }
+        L.ff_up = mat_rows(st, up, ups);
+        L.ff_down = mat_rows(st, up, downs);
+        L.router = up.vec(expect(st, p + "router", rows, W));
+        if (st.contains(p + "correction")) L.moe_correction = up.vec(expect1(st, p + "correction", rows));
+        if (const JsonValue *sh = obj_or_null(f, "shared")) {
+            L.shared_ff = (int32_t)sh->at("ff").num;
+            if (rows_of(st, p + "shared.up") != L.shared_ff || rows_of(st, p + "shared.down") != W) POWERSERVE_ABORT(p + "shared: expert shapes");
+            L.shared_up = mat1(st, up, p + "shared.up");
+            L.shared_down = mat1(st, up, p + "shared.down");
+        }
+    } else {
+        POWERSERVE_ABORT(p + ": feed-forward kind " + kind + " is not known");
+    }
+}
+void pokatar(const JsonValue &cfg, const SafeTensorsFile &st, SeqUploader &up, std::vector<ps_seq_layer> &layers, ps_seq_desc &d) {
+    d.width = (int32_t)cfg.at("width").num;
+    d.vocab = (int32_t)cfg.at("vocab").num;
+    d.canon_taps = 1;
+    d.norm_eps = (float)cfg.at("norm").at("eps").num;
+    d.norm_offset = 0.0f;
+    d.norm_center = 1;
+    d.logit_scale = 1.0f;
+    d.loop_times = 1;
+    d.embed = mat1(st, up, "embed");
+    d.head = d.embed; // the logits are taken against the embedding table itself
+    d.final_norm = up.vec(expect1(st, "final.norm", d.width));
+    const auto &ls = cfg.at("layers").arr;
+    for (size_t i = 0; i < ls.size(); i++) {
+        const JsonValue &lc = ls[i], &mc = lc.at("mixer");
+        const std::string p = "l" + std::to_string(i) + ".", kind = lc.at("type").str;
+        ps_seq_layer L{};
+        L.form = PS_LAYER_PRENORM;
+        L.mix_scale = 1.f;
+        L.norm1 = up.vec(expect1(st, p + "norm1", d.width));
+        if (kind == "attention") sink_attention_mixer(L, st, up, p + "mix.", mc);
+        else if (kind == "latent_attention") shared_key_latent_mixer(L, st, up, p + "mix.", mc);
+        else POWERSERVE_ABORT("layer " + std::to_string(i) + ": mixer type " + kind + " is not known");
+        if (lc.contains("mlp") && lc.at("mlp").kind == JsonValue::OBJ) {
+            L.norm2 = up.vec(expect1(st, p + "norm2", d.width));
+            relu_feed_forward(L, st, up, p + "mlp.", lc.at("mlp"), d.width);
+        }
+        layers.push_back(L);
+    }
+}
 } // namespace
 
 const std::map<std::string, SeqArchitecture> &seq_architectures() {
-    static const std::map<std::string, SeqArchitecture> reg = {{"Ranutar", ranutar}, {"Vobisun", vobisun}, {"Zusolix", zusolix}};
+    static const std::map<std::string, SeqArchitecture> reg = {{"Ranutar", ranutar}, {"Vobisun", vobisun}, {"Zusolix", zusolix}, {"Pokatar", pokatar}};
     return reg;
 }
 bool is_seq_model_dir(const std::string &dir) {

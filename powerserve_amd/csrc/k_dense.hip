@@ -79,6 +79,8 @@ static __device__ __forceinline__ float dn_epi(const dn_args &g, float acc, long
         else acc = g.act_q * (expm1f(acc) - acc) + 0.5f * acc;
     } else if (g.act == PSD_ACT_TANH) {
         acc = tanhf(acc);
+    } else if (g.act == PSD_ACT_RELU2) {
+        acc = acc > 0.f ? acc * acc : 0.f;
     }
     return acc * g.alpha;
 }
@@ -87,10 +89,11 @@ static __device__ __forceinline__ float dn_silu(float x) { return x / (1.f + exp
 // this with both values, only the even row stores).
 static __device__ __forceinline__ void dn_put(const dn_args &g, long long t, long long n, float acc, float other, bool in) {
     const float rs = in && g.out_scale ? g.out_scale[t] : 1.f;
-    if (g.act == PSD_ACT_SILU_PAIR) {
+    if (g.act == PSD_ACT_SILU_PAIR || g.act == PSD_ACT_RELU_PAIR) {
         if (in && !(n & 1)) {
             float *p = g.out + t * g.ldo + (n >> 1);
-            const float v = dn_silu(acc) * other * g.alpha * rs;
+            if (g.bias) { acc += g.bias[n]; other += g.bias[n + 1]; }
+            const float v = (g.act == PSD_ACT_SILU_PAIR ? dn_silu(acc) : fmaxf(acc, 0.f)) * other * g.alpha * rs;
             *p = g.accum ? *p + v : v;
         }
         return;
@@ -315,7 +318,9 @@ __global__ __launch_bounds__(256) void dense_mv_grouped_kernel(dn_args g) {
 #pragma unroll
         for (int q = 0; q < RW; q++) acc[q] = 0.f;
         for (int c = 0; c < inner; c++) {
-            const WT *W = (const WT *)g.w + (long long)g.g_sel[(long long)r * inner + c] * g.wstride;
+            const int sel = g.g_sel[(long long)r * inner + c];
+            if (sel >= g.groups) continue; // (a slot whose choice has no matrix -- an identity expert -- adds nothing here; the same for every lane of the block)
+            const WT *W = (const WT *)g.w + (long long)sel * g.wstride;
             const float *x = xs + (long long)c * Kp;
             if (vec) {
                 for (long long k = (long long)lane * VE; k < K; k += 128 * VE) {
@@ -493,7 +498,7 @@ int psk_dense(hipStream_t st, const psk_dense_args &a) {
         g.g_adiv = a.g_adiv; g.g_odiv = a.g_odiv; g.g_inner = a.g_inner; g.g_sel = a.g_sel; g.g_scale = a.g_scale;
         if (!a.g_list) { // a mat-vec per output row (T rows of g_inner slots each); four rows per wave only where that still leaves about 1024 waves
             const long long waves4 = (g.N + 3) / 4 * a.T;
-            const int RW = waves4 >= 1024 ? 4 : (waves4 >= 512 || g.act == PSD_ACT_SILU_PAIR) ? 2 : 1; // (a gate / up pair sits in one wave)
+            const int RW = waves4 >= 1024 ? 4 : (waves4 >= 512 || g.act == PSD_ACT_SILU_PAIR || g.act == PSD_ACT_RELU_PAIR) ? 2 : 1; // (a gate / up pair sits in one wave)
             const size_t lds = kp4 * a.g_inner;
             if (bf) {
                 if (RW == 4) dn_launch_mv_grouped<unsigned short, 4>(st, g, a.T, lds);

@@ -1,6 +1,7 @@
 // Latent attention of the layer-list models: what a token leaves behind is its normalised key-value latent c (kv_rank numbers) and one rotated
 // key part shared by all heads (rot_dim numbers), kept in a per-sequence RING of `cap` rows (row = position mod cap; cap >= window - 1 + the
-// widest step, so a step never overwrites a row one of its own tokens still sees).  Scores, soft-max and the weighted sum are fp32.
+// widest step, so a step never overwrites a row one of its own tokens still sees).  Scores, soft-max and the weighted sum are fp32.  cos and sin of the
+// rotation may carry a common factor (rot_mag: frequency scaling by wavelength stretches both), and a head's output a sigmoid gate.
 //   latent_prep_kernel   norms of the two latents, rotation of the shared key part, ring append
 //   latent_attn_kernel   one wave per (token, head) over per-head keys / values expanded from the ring rows of the window (the plain form)
 //   latent_attn_mfma_kernel / latent_absorbed_kernel (+ fold, combine, unfold): the matrix-core forms for a portion and for a single token, below
@@ -22,7 +23,7 @@ static __device__ __forceinline__ float la_wave_max(float v) {
 
 __global__ __launch_bounds__(256) void latent_prep_kernel(const ps_seq_step *step, long long ring_off, int cap, const float *y, long long ldy, const float *qnorm,
                                                           const float *kvnorm, float eps, int q_rank, int kv_rank, int rot_dim, int rot_dims, const float *freq, float *cq,
-                                                          long long ldcq) {
+                                                          long long ldcq, float rot_mag) {
     __shared__ float red[8];
     const int t = blockIdx.x, tid = threadIdx.x;
     const long long pos = step->pos0 + t;
@@ -35,13 +36,13 @@ __global__ __launch_bounds__(256) void latent_prep_kernel(const ps_seq_step *ste
     b = la_wave_sum(b);
     if ((tid & 63) == 0) { red[tid >> 6] = a; red[4 + (tid >> 6)] = b; }
     __syncthreads();
-    const float ia = 1.f / sqrtf((red[0] + red[1] + red[2] + red[3]) / (float)q_rank + eps);
+    const float ia = q_rank > 0 ? 1.f / sqrtf((red[0] + red[1] + red[2] + red[3]) / (float)q_rank + eps) : 0.f; // (q_rank 0: the queries do not pass a latent)
     const float ib = 1.f / sqrtf((red[4] + red[5] + red[6] + red[7]) / (float)kv_rank + eps);
     for (int i = tid; i < q_rank; i += 256) cq[(long long)t * ldcq + i] = yt[i] * ia * qnorm[i];
     for (int i = tid; i < kv_rank; i += 256) ring[i] = ckv[i] * ib * kvnorm[i];
     const int half = rot_dims / 2; // the first rot_dims of the part are rotated, pairs (i, i + rot_dims / 2); the rest passes unchanged
     for (int i = tid; i < half; i += 256) {
-        const float ang = (float)pos * freq[i], c = cosf(ang), s = sinf(ang);
+        const float ang = (float)pos * freq[i], c = cosf(ang) * rot_mag, s = sinf(ang) * rot_mag;
         const float u = kr[i], v = kr[i + half];
         ring[kv_rank + i] = u * c - v * s;
         ring[kv_rank + half + i] = v * c + u * s;
@@ -49,16 +50,16 @@ __global__ __launch_bounds__(256) void latent_prep_kernel(const ps_seq_step *ste
     for (int i = 2 * half + tid; i < rot_dim; i += 256) ring[kv_rank + i] = kr[i];
 }
 void psk_latent_prep(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int cap, const float *y, int64_t ldy, const float *qnorm, const float *kvnorm,
-                     float eps, int q_rank, int kv_rank, int rot_dim, int rot_dims, const float *freq, int T, float *cq, int64_t ldcq) {
+                     float eps, int q_rank, int kv_rank, int rot_dim, int rot_dims, const float *freq, int T, float *cq, int64_t ldcq, float rot_mag) {
     hipLaunchKernelGGL(latent_prep_kernel, dim3(T), dim3(256), 0, st, step, (long long)ring_off, cap, y, (long long)ldy, qnorm, kvnorm, eps, q_rank, kv_rank, rot_dim,
-                       rot_dims, freq, cq, (long long)ldcq);
+                       rot_dims, freq, cq, (long long)ldcq, rot_mag);
 }
 
 // dynamic LDS: qs [d + dr], ps [64]
 #define LA_NV 4 // value columns per lane: dv <= 256
 __global__ __launch_bounds__(64) void latent_attn_kernel(const ps_seq_step *step, long long ring_off, int cap, const float *q, long long ldq, const float *kv,
                                                          long long ldkv, const float *freq, int H, int d, int dr, int rot_dims, int dv, int kv_rank, int window,
-                                                         float scale, float *o, long long ldo) {
+                                                         float scale, float *o, long long ldo, float rot_mag, const float *gate, long long ldg) {
     extern __shared__ float lds[];
     float *qs = lds, *ps = lds + d + dr;
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
@@ -70,7 +71,7 @@ __global__ __launch_bounds__(64) void latent_attn_kernel(const ps_seq_step *step
     for (int i = lane; i < d; i += 64) qs[i] = qt[i];
     for (int i = 2 * half + lane; i < dr; i += 64) qs[d + i] = qt[d + i];
     for (int i = lane; i < half; i += 64) {
-        const float ang = (float)p * freq[i], c = cosf(ang), s = sinf(ang);
+        const float ang = (float)p * freq[i], c = cosf(ang) * rot_mag, s = sinf(ang) * rot_mag;
         const float u = qt[d + i], v = qt[d + half + i];
         qs[d + i] = u * c - v * s;
         qs[d + half + i] = v * c + u * s;
@@ -110,15 +111,16 @@ __global__ __launch_bounds__(64) void latent_attn_kernel(const ps_seq_step *step
                 if (lane + 64 * x < dv) acc[x] = fmaf(pk, vr[lane + 64 * x], acc[x]);
         }
     }
-    const float il = 1.f / l;
+    const float il = (gate ? 1.f / (1.f + expf(-gate[(long long)t * ldg + h])) : 1.f) / l;
 #pragma unroll
     for (int x = 0; x < LA_NV; x++)
         if (lane + 64 * x < dv) o[(long long)t * ldo + (long long)h * dv + lane + 64 * x] = acc[x] * il;
 }
 void psk_latent_attn(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int cap, const float *q, int64_t ldq, const float *kv, int64_t ldkv,
-                     const float *freq, int H, int d, int dr, int rot_dims, int dv, int kv_rank, int window, float scale, int T, float *o, int64_t ldo) {
+                     const float *freq, int H, int d, int dr, int rot_dims, int dv, int kv_rank, int window, float scale, int T, float *o, int64_t ldo, float rot_mag,
+                     const float *gate, int64_t ldg) {
     hipLaunchKernelGGL(latent_attn_kernel, dim3(T, H), dim3(64), (size_t)(d + dr + 64) * 4, st, step, (long long)ring_off, cap, q, (long long)ldq, kv, (long long)ldkv,
-                       freq, H, d, dr, rot_dims, dv, kv_rank, window, scale, o, (long long)ldo);
+                       freq, H, d, dr, rot_dims, dv, kv_rank, window, scale, o, (long long)ldo, rot_mag, gate, (long long)ldg);
 }
 
 // ---------------------------------------------------------------------------------------------------- matrix-core form
@@ -137,7 +139,7 @@ void psk_latent_attn(hipStream_t st, const ps_seq_step *step, int64_t ring_off, 
 template <int NJ>
 __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(const ps_seq_step *step, long long ring_off, int cap, const float *q, long long ldq, const float *kv,
                                                                long long ldkv, const float *freq, int H, int d, int dr, int rot_dims, int dv, int kv_rank, int window,
-                                                               float scale, int T, float *o, long long ldo) {
+                                                               float scale, int T, float *o, long long ldo, float rot_mag, const float *gate, long long ldg) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 15, lq = lane >> 4, h = blockIdx.y;
     const int qld = d + dr + 4;
@@ -156,7 +158,7 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(const ps_seq_step
         for (int c = lane; c < d; c += 64) qr[c] = in ? qt[c] : 0.f;
         for (int c = 2 * half + lane; c < dr; c += 64) qr[d + c] = in ? qt[d + c] : 0.f;
         for (int i = lane; i < half; i += 64) {
-            const float ang = (float)(pos0 + t) * freq[i], cs = cosf(ang), sn = sinf(ang);
+            const float ang = (float)(pos0 + t) * freq[i], cs = cosf(ang) * rot_mag, sn = sinf(ang) * rot_mag;
             const float u = in ? qt[d + i] : 0.f, v = in ? qt[d + half + i] : 0.f;
             qr[d + i] = u * cs - v * sn;
             qr[d + half + i] = v * cs + u * sn;
@@ -188,7 +190,7 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(const ps_seq_step
         for (int i = 0; i < 4; i++) { // a lane's four tiles of a 64-column group are four consecutive columns: one 16-byte store
             const int t = t0 + 4 * lq + i, c = 64 * J + 4 * lr;
             if (t < T && c < dv) {
-                const float il = 1.f / l[i];
+                const float il = (gate ? 1.f / (1.f + expf(-gate[(long long)t * ldg + h])) : 1.f) / l[i];
                 *(la_f4 *)(o + (long long)t * ldo + (long long)h * dv + c) = la_f4{acc[4 * J][i] * il, acc[4 * J + 1][i] * il, acc[4 * J + 2][i] * il, acc[4 * J + 3][i] * il};
             }
         }
@@ -196,12 +198,13 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(const ps_seq_step
 
 bool psk_latent_attn_mfma_ok(int d, int dr, int dv) { return d % 16 == 0 && dr % 16 == 0 && dv % 4 == 0 && dv <= 128 && (size_t)4 * (16 * (d + dr + 4) + 16 * 17) * 4 <= 160 * 1024; }
 void psk_latent_attn_mfma(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int cap, const float *q, int64_t ldq, const float *kv, int64_t ldkv,
-                          const float *freq, int H, int d, int dr, int rot_dims, int dv, int kv_rank, int window, float scale, int T, float *o, int64_t ldo) {
+                          const float *freq, int H, int d, int dr, int rot_dims, int dv, int kv_rank, int window, float scale, int T, float *o, int64_t ldo, float rot_mag,
+                          const float *gate, int64_t ldg) {
     const size_t lds = (size_t)4 * (16 * (d + dr + 4) + 16 * 17) * 4;
     static unsigned long long mask = 0;
     if (ps_first_on_device(&mask)) (void)hipFuncSetAttribute((const void *)latent_attn_mfma_kernel<8>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     hipLaunchKernelGGL(latent_attn_mfma_kernel<8>, dim3((T + 63) / 64, H), dim3(256), lds, st, step, (long long)ring_off, cap, q, (long long)ldq, kv, (long long)ldkv, freq,
-                       H, d, dr, rot_dims, dv, kv_rank, window, scale, T, o, (long long)ldo);
+                       H, d, dr, rot_dims, dv, kv_rank, window, scale, T, o, (long long)ldo, rot_mag, gate, (long long)ldg);
 }
 
 // ---------------------------------------------------------------------------------------------------- single token, absorbed
@@ -227,7 +230,7 @@ __global__ __launch_bounds__(256) void latent_fold_q_kernel(const float *q, int 
 }
 // o[h][x] = sum_r Wuv[h * dv + x][r] ol[h][r]: the value expansion of the attended latent.  A wave per output row.
 template <typename WT>
-__global__ __launch_bounds__(256) void latent_unfold_v_kernel(const float *ol, const WT *wuv, int dv, int R, int rows, float *o) {
+__global__ __launch_bounds__(256) void latent_unfold_v_kernel(const float *ol, const WT *wuv, int dv, int R, int rows, float *o, const float *gate) {
     const int row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
     if (row >= rows) return;
     const float *x = ol + (long long)(row / dv) * R;
@@ -239,14 +242,14 @@ __global__ __launch_bounds__(256) void latent_unfold_v_kernel(const float *ol, c
         a = fmaf(w, x[r], a);
     }
     a = la_wave_sum(a);
-    if (lane == 0) o[row] = a;
+    if (lane == 0) o[row] = gate ? a / (1.f + expf(-gate[row / dv])) : a; // (the head's output gate)
 }
 
 // rows = heads (16 per block), keys = ring rows; wave w of block (split s, head tile) takes key tile 4 s + w of the window.  Partials:
 // per (key tile, head) R unnormalised outputs, then m and l.  dynamic LDS: 16 x qld + 4 x 16 x 17
 template <int NJ>
 __global__ __launch_bounds__(256) void latent_absorbed_kernel(const ps_seq_step *step, long long ring_off, int cap, const float *qa, const float *q, int qstride, int d,
-                                                              int dr, int rot_dims, const float *freq, int H, int R, int window, float scale, float *part) {
+                                                              int dr, int rot_dims, const float *freq, int H, int R, int window, float scale, float *part, float rot_mag) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 15, lq = lane >> 4, h0 = blockIdx.y * 16;
     const int qld = R + dr + 4;
@@ -262,7 +265,7 @@ __global__ __launch_bounds__(256) void latent_absorbed_kernel(const ps_seq_step 
         for (int c = 2 * half + lane; c < dr; c += 64) qr[R + c] = h < H ? q[(long long)h * qstride + d + c] : 0.f;
     }
     for (int i = lane; i < half; i += 64) {
-        const float ang = (float)p * freq[i], cs = cosf(ang), sn = sinf(ang);
+        const float ang = (float)p * freq[i], cs = cosf(ang) * rot_mag, sn = sinf(ang) * rot_mag;
         for (int r = wave; r < 16; r += 4) {
             const int h = h0 + r;
             const float *qt = q + (long long)(h < H ? h : 0) * qstride + d;
@@ -335,7 +338,7 @@ bool psk_latent_absorbed_ok(int d, int dr, int dv, int R) { return R % 16 == 0 &
 size_t psk_latent_absorbed_scratch(int H, int R, int window) { return ((size_t)((window + 15) / 16 + 4) * H * (R + 4) + (size_t)2 * H * R) * 4; }
 // q [H][d + dr] (row stride qstride) -> o [H * dv]; ukv: rows uk | uv of the expansion matrix [H d + H dv][R]; scratch from psk_latent_absorbed_scratch
 void psk_latent_absorbed(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int cap, const float *q, int qstride, const ps_dense *ukv, const float *freq,
-                         int H, int d, int dr, int rot_dims, int dv, int R, int window, float scale, float *scratch, float *o) {
+                         int H, int d, int dr, int rot_dims, int dv, int R, int window, float scale, float *scratch, float *o, float rot_mag, const float *gate) {
     const int max_tiles = (window + 15) / 16 + 1; // (a window that does not start on a tile's edge touches one tile more)
     float *qa = scratch, *ol = qa + (size_t)H * R, *part = ol + (size_t)H * R;
     const bool bf = ukv->dtype == PS_BF16;
@@ -346,14 +349,14 @@ void psk_latent_absorbed(hipStream_t st, const ps_seq_step *step, int64_t ring_o
     if (R <= 128) {
         static unsigned long long mask = 0;
         if (ps_first_on_device(&mask)) (void)hipFuncSetAttribute((const void *)latent_absorbed_kernel<8>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        hipLaunchKernelGGL(latent_absorbed_kernel<8>, grid, dim3(256), lds, st, step, (long long)ring_off, cap, qa, q, qstride, d, dr, rot_dims, freq, H, R, window, scale, part);
+        hipLaunchKernelGGL(latent_absorbed_kernel<8>, grid, dim3(256), lds, st, step, (long long)ring_off, cap, qa, q, qstride, d, dr, rot_dims, freq, H, R, window, scale, part, rot_mag);
     } else {
         static unsigned long long mask = 0;
         if (ps_first_on_device(&mask)) (void)hipFuncSetAttribute((const void *)latent_absorbed_kernel<32>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        hipLaunchKernelGGL(latent_absorbed_kernel<32>, grid, dim3(256), lds, st, step, (long long)ring_off, cap, qa, q, qstride, d, dr, rot_dims, freq, H, R, window, scale, part);
+        hipLaunchKernelGGL(latent_absorbed_kernel<32>, grid, dim3(256), lds, st, step, (long long)ring_off, cap, qa, q, qstride, d, dr, rot_dims, freq, H, R, window, scale, part, rot_mag);
     }
     hipLaunchKernelGGL(latent_combine_kernel, dim3(H), dim3(256), (size_t)grid.x * 4 * 4, st, step, part, H, R, window, (int)grid.x * 4, ol);
     const int rows = H * dv;
-    if (bf) hipLaunchKernelGGL(latent_unfold_v_kernel<unsigned short>, dim3((rows + 3) / 4), dim3(256), 0, st, ol, (const unsigned short *)ukv->data + (size_t)H * d * R, dv, R, rows, o);
-    else hipLaunchKernelGGL(latent_unfold_v_kernel<float>, dim3((rows + 3) / 4), dim3(256), 0, st, ol, (const float *)ukv->data + (size_t)H * d * R, dv, R, rows, o);
+    if (bf) hipLaunchKernelGGL(latent_unfold_v_kernel<unsigned short>, dim3((rows + 3) / 4), dim3(256), 0, st, ol, (const unsigned short *)ukv->data + (size_t)H * d * R, dv, R, rows, o, gate);
+    else hipLaunchKernelGGL(latent_unfold_v_kernel<float>, dim3((rows + 3) / 4), dim3(256), 0, st, ol, (const float *)ukv->data + (size_t)H * d * R, dv, R, rows, o, gate);
 }

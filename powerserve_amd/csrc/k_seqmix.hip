@@ -43,11 +43,12 @@ void psk_rmsnorm(hipStream_t st, const float *x, int64_t ldx, const int32_t *idx
 // The front of a parallel layer without an input filter, one block per row:  x = sum_j mix[j] X_j  over the nmix streams X_j = src + j stride (mix NULL: the last
 // of them as it is), kept in xout (NULL: not kept; it may be the last stream itself); then, over `groups` equal parts of the row each with its own mean square,
 // h = x / rms * (offset + w1) and h2 = x / rms * (offset + w2): two norms of the same vector share their statistics (w1 / w2 NULL: not wanted).
-// dynamic LDS: n + groups floats.
+// center: a layer norm instead -- the part's mean is taken off and the variance is the mean of the squared deviations (two passes over the row in LDS).
+// dynamic LDS: n + 2 groups floats.
 __global__ __launch_bounds__(1024) void sq_front_kernel(const float *src, long long stride, int nmix, const float *mix, const int32_t *idx, float *xout, const float *w1,
-                                                       float *h, const float *w2, float *h2, int groups, float offset, float eps, long long n) {
+                                                       float *h, const float *w2, float *h2, int groups, float offset, float eps, long long n, int center) {
     extern __shared__ float fr[];
-    float *xs = fr, *inv = fr + n;
+    float *xs = fr, *inv = fr + n, *mean = inv + groups;
     const long long r = idx ? idx[blockIdx.x] : blockIdx.x, o = (long long)blockIdx.x * n;
     const int tid = threadIdx.x, nt = blockDim.x;
     for (long long i = tid; i < n; i += nt) {
@@ -65,26 +66,33 @@ __global__ __launch_bounds__(1024) void sq_front_kernel(const float *src, long l
     __syncthreads();
     const long long gs = n / groups;
     for (int g = tid >> 6; g < groups; g += nt >> 6) {
+        float mu = 0.f;
+        if (center) {
+            for (long long i = tid & 63; i < gs; i += 64) mu += xs[g * gs + i];
+#pragma unroll
+            for (int o2 = 32; o2 > 0; o2 >>= 1) mu += __shfl_xor(mu, o2, 64);
+            mu /= (float)gs;
+        }
         float s = 0.f;
-        for (long long i = tid & 63; i < gs; i += 64) s += xs[g * gs + i] * xs[g * gs + i];
+        for (long long i = tid & 63; i < gs; i += 64) { const float dv = xs[g * gs + i] - mu; s += dv * dv; }
 #pragma unroll
         for (int o2 = 32; o2 > 0; o2 >>= 1) s += __shfl_xor(s, o2, 64);
-        if ((tid & 63) == 0) inv[g] = 1.f / sqrtf(s / (float)gs + eps);
+        if ((tid & 63) == 0) { inv[g] = 1.f / sqrtf(s / (float)gs + eps); mean[g] = mu; }
     }
     __syncthreads();
     for (long long i = tid; i < n; i += nt) {
-        const float v = xs[i] * inv[i / gs];
+        const float v = (xs[i] - mean[i / gs]) * inv[i / gs];
         if (w1) h[o + i] = v * (offset + w1[i]);
         if (w2) h2[o + i] = v * (offset + w2[i]);
     }
 }
 void psk_front(hipStream_t st, const float *src, int64_t stride, int nmix, const float *mix, const int32_t *idx, float *xout, const float *w1, float *h, const float *w2,
-               float *h2, int groups, float offset, float eps, int64_t n, int rows) {
+               float *h2, int groups, float offset, float eps, int64_t n, int rows, int center) {
     if (rows <= 0) return;
     static unsigned long long mask = 0;
     if (ps_first_on_device(&mask)) (void)hipFuncSetAttribute((const void *)sq_front_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    hipLaunchKernelGGL(sq_front_kernel, dim3(rows), dim3(rows <= 8 && n >= 2048 ? 1024 : 256), (size_t)(n + groups) * 4, st, src, (long long)stride, nmix, mix, idx, xout, w1, h, w2, h2, groups, offset, eps,
-                       (long long)n);
+    hipLaunchKernelGGL(sq_front_kernel, dim3(rows), dim3(rows <= 8 && n >= 2048 ? 1024 : 256), (size_t)(n + 2 * groups) * 4, st, src, (long long)stride, nmix, mix, idx, xout, w1, h, w2, h2, groups, offset, eps,
+                       (long long)n, center);
 }
 
 __global__ __launch_bounds__(256) void sq_norm_residual_kernel(float *x, const float *y, const float *w, float offset, float eps, long long n) {

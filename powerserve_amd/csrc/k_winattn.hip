@@ -1,7 +1,8 @@
 // Windowed attention with pooled blocks of the layer-list models (PS_MIX_WINATTN): grouped-query soft-max attention in which a token at
 // position p sees the `window` positions up to itself and, beside them, ONE key and value for every block of `pool` consecutive positions that
 // lies wholly before that window (the means of the block's keys / values as the ring holds them); a per-head sink adds exp(sink) to the
-// denominator, a per-head temperature multiplies the scores, a per-head sigmoid gate the output.  What a sequence keeps: a RING of the last
+// denominator, a per-head temperature multiplies the scores, a sigmoid gate (per head, or element by element) the output; the q / k norms are taken over
+// the whole projection or per head, and a head's value may be made a unit-rms vector as it is cached.  What a sequence keeps: a RING of the last
 // `cap` tokens' keys and values (row = position mod cap; cap >= window - 1 + the widest step) and the block means, one row per block, which
 // grow with the sequence.  Scores, soft-max and the weighted sums are fp32.
 //   winattn_prep_kernel    norms over the whole q / k projections, rotation, ring append            (one or a few blocks per token)
@@ -36,12 +37,14 @@ static __device__ __forceinline__ long long wa_blocks(long long p, int window, i
 // winattn_pool_kernel makes for a portion).  dynamic LDS: rot_dims floats (cos | sin of the token's angles, shared by all heads).
 __global__ __launch_bounds__(256) void winattn_prep_kernel(const ps_seq_step *step, long long ring_off, int cap, long long pool_off, int pool, const float *y,
                                                            long long ldy, const float *qnorm, const float *knorm, float eps, int H, int G, int d, int dv, int rot_dims,
-                                                           int pairing, const float *freq, float *qo, long long ldq, float qt_coef, int qt_every) {
+                                                           int pairing, const float *freq, float *qo, long long ldq, float qt_coef, int qt_every, int head_norm,
+                                                           int v_unit) {
     extern __shared__ float cs[];
     __shared__ float red[8];
     const int t = blockIdx.x, tid = threadIdx.x;
     const long long pos = step->pos0 + t;
     const int nq = H * d, nk = G * d, nv = G * dv, half = rot_dims / 2;
+    float *hinv = cs + rot_dims + 2; // per-head norms: 1 / rms of every q head, k head, v head ([H | G | G])
     const float *qt = y + (long long)t * ldy, *kt = qt + nq, *vt = kt + nk;
     float *ring = step->state + ring_off + (pos % cap) * (long long)(nk + nv);
     // a query temperature that grows with the position in steps of qt_every tokens: 1 + coef ln(floor((pos + 1) / every) + 1)
@@ -52,17 +55,30 @@ __global__ __launch_bounds__(256) void winattn_prep_kernel(const ps_seq_step *st
         cs[half + i] = sinf(ang);
     }
     float a = 0.f, b = 0.f;
-    if (qnorm) for (int i = tid; i < nq; i += 256) a += qt[i] * qt[i];
-    if (knorm) for (int i = tid; i < nk; i += 256) b += kt[i] * kt[i];
+    if (qnorm && !head_norm) for (int i = tid; i < nq; i += 256) a += qt[i] * qt[i];
+    if (knorm && !head_norm) for (int i = tid; i < nk; i += 256) b += kt[i] * kt[i];
     a = wa_wave_sum(a);
     b = wa_wave_sum(b);
     if ((tid & 63) == 0) { red[tid >> 6] = a; red[4 + (tid >> 6)] = b; }
+    if (head_norm || v_unit) { // a wave per head: heads 0 .. H - 1 of q, then G of k, then G of v
+        for (int hd = tid >> 6; hd < H + 2 * G; hd += 4) {
+            const bool isq = hd < H, isk = !isq && hd < H + G;
+            const float *src = isq ? qt + hd * d : isk ? kt + (hd - H) * d : vt + (hd - H - G) * dv;
+            const int n = isq || isk ? d : dv;
+            const bool on = isq ? (head_norm && qnorm) : isk ? (head_norm && knorm) : v_unit != 0;
+            float ss = 0.f;
+            if (on) for (int i = tid & 63; i < n; i += 64) ss += src[i] * src[i];
+            ss = wa_wave_sum(ss);
+            if ((tid & 63) == 0) hinv[hd] = on ? 1.f / sqrtf(ss / (float)n + eps) : 1.f;
+        }
+    }
     __syncthreads();
-    const float ia = qnorm ? 1.f / sqrtf((red[0] + red[1] + red[2] + red[3]) / (float)nq + eps) : 1.f;
-    const float ib = knorm ? 1.f / sqrtf((red[4] + red[5] + red[6] + red[7]) / (float)nk + eps) : 1.f;
+    const float ia = qnorm && !head_norm ? 1.f / sqrtf((red[0] + red[1] + red[2] + red[3]) / (float)nq + eps) : 1.f;
+    const float ib = knorm && !head_norm ? 1.f / sqrtf((red[4] + red[5] + red[6] + red[7]) / (float)nk + eps) : 1.f;
     // element i of a projection (c = its index in its head): normed, and where c < rot_dims turned together with its partner
-    auto turned = [&](const float *src, const float *w, float inv, int i) {
+    auto turned = [&](const float *src, const float *w, float inv, const float *hi, int i) {
         const int c = i % d;
+        if (head_norm) { inv = hi[i / d]; if (w) w += c - i; } // (the head's own statistics; one weight vector for every head: w[i] below reads w[c])
         const float self = src[i] * inv * (w ? w[i] : 1.f);
         if (c >= 2 * half) return self;
         int partner, pair;
@@ -84,10 +100,10 @@ __global__ __launch_bounds__(256) void winattn_prep_kernel(const ps_seq_step *st
     // the elements of q | k | v are spread over the blocks of a token (gridDim.y; every block has made the sums above for itself)
     for (int e = blockIdx.y * 256 + tid; e < nq + nk + nv; e += 256 * gridDim.y) {
         if (e < nq) {
-            qo[(long long)t * ldq + e] = turned(qt, qnorm, ia, e) * qtemp;
+            qo[(long long)t * ldq + e] = turned(qt, qnorm, ia, hinv, e) * qtemp;
         } else {
             const int i = e - nq;
-            const float v = i < nk ? turned(kt, knorm, ib, i) : vt[i - nk];
+            const float v = i < nk ? turned(kt, knorm, ib, hinv + H, i) : (v_unit ? vt[i - nk] * hinv[H + G + (i - nk) / dv] : vt[i - nk]);
             ring[i] = v;
             pooled(i, v);
         }
@@ -111,11 +127,11 @@ __global__ __launch_bounds__(256) void winattn_pool_kernel(const ps_seq_step *st
 
 void psk_winattn_prep(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int cap, int64_t pool_off, int pool, const float *y, int64_t ldy, const float *qnorm,
                       const float *knorm, float eps, int H, int G, int d, int dv, int rot_dims, int pairing, const float *freq, int T, float *q, int64_t ldq, float qt_coef,
-                      int qt_every) {
+                      int qt_every, int head_norm, int v_unit) {
     const int total = H * d + G * (d + dv);
     const int split = T >= 64 ? 1 : std::min(16, (total + 511) / 512); // few tokens: a token's elements over several blocks
-    hipLaunchKernelGGL(winattn_prep_kernel, dim3(T, split), dim3(256), (size_t)(rot_dims + 2) * 4, st, step, (long long)ring_off, cap, (long long)pool_off, pool, y, (long long)ldy,
-                       qnorm, knorm, eps, H, G, d, dv, rot_dims, pairing, freq, q, (long long)ldq, qt_coef, qt_every);
+    hipLaunchKernelGGL(winattn_prep_kernel, dim3(T, split), dim3(256), (size_t)(rot_dims + 2 + H + 2 * G) * 4, st, step, (long long)ring_off, cap, (long long)pool_off, pool, y,
+                       (long long)ldy, qnorm, knorm, eps, H, G, d, dv, rot_dims, pairing, freq, q, (long long)ldq, qt_coef, qt_every, head_norm, v_unit);
     if (pool > 0 && T > 1) {
         const int rs = G * (d + dv);
         hipLaunchKernelGGL(winattn_pool_kernel, dim3((rs + 255) / 256, (T - 1) / pool + 2), dim3(256), 0, st, step, (long long)ring_off, cap, (long long)pool_off, pool, rs);
@@ -134,7 +150,7 @@ static __device__ __forceinline__ float wa_sigmoid(float x) { return 1.f / (1.f 
 #define WA_NV 4 // value columns per lane: dv <= 256
 __global__ __launch_bounds__(64) void winattn_kernel(const ps_seq_step *step, long long ring_off, int cap, long long pool_off, int pool, const float *q, long long ldq,
                                                      const float *gate, long long ldg, const float *temp, const float *sink, int H, int G, int d, int dv, int window,
-                                                     float scale, float *o, long long ldo, float softcap) {
+                                                     float scale, float *o, long long ldo, float softcap, int gate_elem) {
     extern __shared__ float lds[];
     float *qs = lds, *ps = lds + d;
     const int t = blockIdx.x, h = blockIdx.y, g = h / (H / G), lane = threadIdx.x;
@@ -177,15 +193,19 @@ __global__ __launch_bounds__(64) void winattn_kernel(const ps_seq_step *step, lo
                 if (lane + 64 * x < dv) acc[x] = fmaf(pk, vr[lane + 64 * x], acc[x]);
         }
     }
-    const float f = wa_finish(m, l, sink, h) * (gate ? wa_sigmoid(gate[(long long)t * ldg + h]) : 1.f);
+    const float f = wa_finish(m, l, sink, h) * (gate && !gate_elem ? wa_sigmoid(gate[(long long)t * ldg + h]) : 1.f);
 #pragma unroll
     for (int x = 0; x < WA_NV; x++)
-        if (lane + 64 * x < dv) o[(long long)t * ldo + (long long)h * dv + lane + 64 * x] = acc[x] * f;
+        if (lane + 64 * x < dv) {
+            const long long c = (long long)h * dv + lane + 64 * x;
+            o[(long long)t * ldo + c] = acc[x] * f * (gate && gate_elem ? wa_sigmoid(gate[(long long)t * ldg + c]) : 1.f);
+        }
 }
 void psk_winattn(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int cap, int64_t pool_off, int pool, const float *q, int64_t ldq, const float *gate,
-                 int64_t ldg, const float *temp, const float *sink, int H, int G, int d, int dv, int window, float scale, int T, float *o, int64_t ldo, float softcap) {
+                 int64_t ldg, const float *temp, const float *sink, int H, int G, int d, int dv, int window, float scale, int T, float *o, int64_t ldo, float softcap,
+                 int gate_elem) {
     hipLaunchKernelGGL(winattn_kernel, dim3(T, H), dim3(64), (size_t)(d + 64) * 4, st, step, (long long)ring_off, cap, (long long)pool_off, pool, q, (long long)ldq, gate,
-                       (long long)ldg, temp, sink, H, G, d, dv, window, scale, o, (long long)ldo, softcap);
+                       (long long)ldg, temp, sink, H, G, d, dv, window, scale, o, (long long)ldo, softcap, gate_elem);
 }
 
 // ---------------------------------------------------------------------------------------------------- matrix-core forms (ps_attn_dev.h)
@@ -194,7 +214,7 @@ void psk_winattn(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int 
 template <int NJ>
 __global__ __launch_bounds__(256) void winattn_mfma_kernel(const ps_seq_step *step, long long ring_off, int cap, long long pool_off, int pool, const float *q, long long ldq,
                                                            const float *gate, long long ldg, const float *temp, const float *sink, int H, int G, int d, int dv, int window,
-                                                           float scale, int T, float *o, long long ldo, float softcap) {
+                                                           float scale, int T, float *o, long long ldo, float softcap, int gate_elem) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 15, lq = lane >> 4, h = blockIdx.y, g = h / (H / G);
     const int qld = d + 4;
@@ -241,11 +261,18 @@ __global__ __launch_bounds__(256) void winattn_mfma_kernel(const ps_seq_step *st
     for (int i = 0; i < 4; i++) {
         const int t = t0 + 4 * lq + i;
         if (t >= T) continue;
-        const float f = wa_finish(m[i], l[i], sink, h) * (gate ? wa_sigmoid(gate[(long long)t * ldg + h]) : 1.f);
+        const float f = wa_finish(m[i], l[i], sink, h) * (gate && !gate_elem ? wa_sigmoid(gate[(long long)t * ldg + h]) : 1.f);
 #pragma unroll
         for (int J = 0; J < NJ / 4; J++) { // a lane's four tiles of a 64-column group are four consecutive columns: one 16-byte store
             const int c = 64 * J + 4 * lr;
-            if (c < dv) *(la_f4 *)(o + (long long)t * ldo + (long long)h * dv + c) = la_f4{acc[4 * J][i] * f, acc[4 * J + 1][i] * f, acc[4 * J + 2][i] * f, acc[4 * J + 3][i] * f};
+            if (c >= dv) continue;
+            la_f4 r = la_f4{acc[4 * J][i] * f, acc[4 * J + 1][i] * f, acc[4 * J + 2][i] * f, acc[4 * J + 3][i] * f};
+            if (gate && gate_elem) {
+                const float *gp = gate + (long long)t * ldg + (long long)h * dv + c;
+#pragma unroll
+                for (int e = 0; e < 4; e++) r[e] *= wa_sigmoid(gp[e]);
+            }
+            *(la_f4 *)(o + (long long)t * ldo + (long long)h * dv + c) = r;
         }
     }
 }
@@ -254,11 +281,12 @@ static size_t wa_mfma_lds(int d) { return (size_t)4 * (16 * (d + 4) + 16 * 17) *
 // the sizes the matrix-core forms take: 16-byte pieces of keys (d a multiple of 16) and values (dv of 4, at most 128 columns per head)
 bool psk_winattn_mfma_ok(int d, int dv) { return d % 16 == 0 && dv % 4 == 0 && dv <= 128 && wa_mfma_lds(d) <= 160 * 1024; }
 void psk_winattn_mfma(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int cap, int64_t pool_off, int pool, const float *q, int64_t ldq, const float *gate,
-                      int64_t ldg, const float *temp, const float *sink, int H, int G, int d, int dv, int window, float scale, int T, float *o, int64_t ldo, float softcap) {
+                      int64_t ldg, const float *temp, const float *sink, int H, int G, int d, int dv, int window, float scale, int T, float *o, int64_t ldo, float softcap,
+                      int gate_elem) {
     static unsigned long long mask = 0;
     if (ps_first_on_device(&mask)) (void)hipFuncSetAttribute((const void *)winattn_mfma_kernel<8>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     hipLaunchKernelGGL(winattn_mfma_kernel<8>, dim3((T + 63) / 64, H), dim3(256), wa_mfma_lds(d), st, step, (long long)ring_off, cap, (long long)pool_off, pool, q,
-                       (long long)ldq, gate, (long long)ldg, temp, sink, H, G, d, dv, window, scale, T, o, (long long)ldo, softcap);
+                       (long long)ldq, gate, (long long)ldg, temp, sink, H, G, d, dv, window, scale, T, o, (long long)ldo, softcap, gate_elem);
 }
 
 // A single token.  Rows = the heads that share key / value group g (16 per block); the keys are cut into tiles of 16 in one index space -- tiles
@@ -310,7 +338,7 @@ __global__ __launch_bounds__(256) void winattn_step_kernel(const ps_seq_step *st
 }
 // o[h][c] = gate_h * sum_tiles exp(m_t - M) o_t[c] / (sum_tiles exp(m_t - M) l_t + exp(sink_h - M)),  M = max(max_t m_t, sink_h)
 __global__ __launch_bounds__(256) void winattn_merge_kernel(const ps_seq_step *step, const float *part, const float *gate, const float *sink, int pool, int H, int dv,
-                                                            int window, int max_tiles, float *o) {
+                                                            int window, int max_tiles, float *o, int gate_elem) {
     extern __shared__ float wts[]; // [max_tiles] weights exp(m_t - M)
     __shared__ float red[4];
     const int h = blockIdx.x, tid = threadIdx.x, dvp = dv + 4;
@@ -335,12 +363,12 @@ __global__ __launch_bounds__(256) void winattn_merge_kernel(const ps_seq_step *s
     if ((tid & 63) == 0) red[tid >> 6] = ls;
     __syncthreads();
     const float L = red[0] + red[1] + red[2] + red[3] + (sink ? expf(sink[h] - M) : 0.f);
-    const float f = (gate ? wa_sigmoid(gate[h]) : 1.f) / L;
+    const float f = (gate && !gate_elem ? wa_sigmoid(gate[h]) : 1.f) / L;
     for (int c = tid; c < dv; c += 256) {
         float a = 0.f;
 #pragma unroll 8
         for (int t = 0; t < nt; t++) a = fmaf(wts[t], part[((long long)t * H + h) * dvp + c], a);
-        o[(long long)h * dv + c] = a * f;
+        o[(long long)h * dv + c] = a * f * (gate && gate_elem ? wa_sigmoid(gate[(long long)h * dv + c]) : 1.f);
     }
 }
 
@@ -353,12 +381,12 @@ size_t psk_winattn_step_scratch(int H, int dv, int window, int pool, int64_t max
 }
 // q [H * d] -> o [H * dv]; gate [H] raw or NULL; scratch from psk_winattn_step_scratch
 void psk_winattn_step(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int cap, int64_t pool_off, int pool, const float *q, const float *gate, const float *temp,
-                      const float *sink, int H, int G, int d, int dv, int window, float scale, int64_t max_context, float *scratch, float *o, float softcap) {
+                      const float *sink, int H, int G, int d, int dv, int window, float scale, int64_t max_context, float *scratch, float *o, float softcap, int gate_elem) {
     const int max_tiles = wa_max_tiles(window, pool, max_context);
     const size_t lds = (size_t)(16 * (d + 4) + 4 * 16 * 17) * 4;
     static unsigned long long mask = 0;
     if (ps_first_on_device(&mask)) (void)hipFuncSetAttribute((const void *)winattn_step_kernel<8>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     const dim3 grid((max_tiles + 3) / 4, (H / G + 15) / 16, G);
     hipLaunchKernelGGL(winattn_step_kernel<8>, grid, dim3(256), lds, st, step, (long long)ring_off, cap, (long long)pool_off, pool, q, temp, H, G, d, dv, window, scale, scratch, softcap);
-    hipLaunchKernelGGL(winattn_merge_kernel, dim3(H), dim3(256), (size_t)grid.x * 4 * 4, st, step, scratch, gate, sink, pool, H, dv, window, (int)grid.x * 4, o);
+    hipLaunchKernelGGL(winattn_merge_kernel, dim3(H), dim3(256), (size_t)grid.x * 4 * 4, st, step, scratch, gate, sink, pool, H, dv, window, (int)grid.x * 4, o, gate_elem);
 }

@@ -21,7 +21,9 @@ struct ps_seq_step {
 };
 
 enum { PSD_ACT_NONE = 0, PSD_ACT_XIELU = 1, PSD_ACT_TANH = 2,
-       PSD_ACT_SILU_PAIR = 3 }; // rows 2i / 2i + 1 of W are a gate and its partner: out[t][i] = silu(row 2i) * (row 2i + 1), N / 2 outputs
+       PSD_ACT_SILU_PAIR = 3,   // rows 2i / 2i + 1 of W are a gate and its partner: out[t][i] = silu(row 2i) * (row 2i + 1), N / 2 outputs (bias: one per row, added first)
+       PSD_ACT_RELU_PAIR = 4,   // the same with relu on the gate
+       PSD_ACT_RELU2 = 5 };     // max(z, 0)^2
 
 // out[t][n] = alpha * act(sum_k A(t, k) W[n][k] + bias[n]),  t < T
 //   A(t, k) = a[row(t)][k], row(t) = t, or (a_row0 + t) mod a_mod when a_mod > 0 (rows of a ring), or, where a_step is given, rows of the
@@ -72,7 +74,8 @@ void psk_norm_residual(hipStream_t st, float *x, const float *y, const float *w,
 // the last stream alone), row(r) = idx ? idx[r] : r, stored to xout[r] (NULL: not kept); then h[r] = norm(x) (offset + w1) and h2[r] = norm(x) (offset + w2) with
 // the norm taken over `groups` parts -- two norms of one vector share their statistics.  w1 / w2 NULL: that output is not made.
 void psk_front(hipStream_t st, const float *src, int64_t stride, int nmix, const float *mix, const int32_t *idx, float *xout, const float *w1, float *h, const float *w2,
-               float *h2, int groups, float offset, float eps, int64_t n, int rows);
+               float *h2, int groups, float offset, float eps, int64_t n, int rows,
+               int center = 0); // 1: layer norms -- (x - mean) / sqrt(mean((x - mean)^2) + eps) over each part
 // Element-wise gated recurrence.  y[t] = [ z | u | g ] (C each): S <- (1 - sigmoid(z)) S + sigmoid(z) c(u), c(u) = sigmoid(u) for negative u, else u + 0.5;
 // o[t] = S silu(g).  State [C] fp32 at step->state + state_off.
 void psk_mingru_scan(hipStream_t st, const ps_seq_step *step, int64_t state_off, const float *y, int64_t ldy, int64_t C, int T, float *o, int64_t ldo);
@@ -106,34 +109,40 @@ void psk_delta_scan(hipStream_t st, const ps_seq_step *step, int64_t state_off, 
 void psk_headnorm_gate(hipStream_t st, float *o, int64_t ldo, const float *g, int64_t ldg, const float *w, int w_stride, float eps, int H, int dv, int T);
 
 // ---- k_moe.hip
-// Router of a mixture of experts, fp32: scores = sigmoid(router h[t]); the `top` largest (ties: the lower index) -> sel[t top + i], wgt[t top + i] (their scores,
-// divided by their sum where norm_top); sgate[t] = sigmoid(shared_gate . h[t]) where shared_gate is given.
+// Router of a mixture of experts, fp32: scores = sigmoid(router h[t]), or (softmax) the soft-max over all `experts` rows; choice scores = scores + correction (NULL: none);
+// with n_groups > 0 only rows of the `keep` groups (equal runs of neighbours) with the largest best choice score stay in the race; the `top` largest choice scores
+// (ties: the lower index) -> sel[t top + i], wgt[t top + i] (their SCORES, divided by their sum where norm_top); sgate[t] = sigmoid(shared_gate . h[t]) where given.
 void psk_moe_route(hipStream_t st, const float *h, int64_t ldh, const float *router, const float *shared_gate, int experts, int top, int norm_top, int64_t K, int T,
-                   int32_t *sel, float *wgt, float *sgate);
+                   int32_t *sel, float *wgt, float *sgate, int softmax = 0, const float *correction = nullptr, int n_groups = 0, int keep = 0);
 // The S slots sorted by expert: seg [experts + 1] (slots of expert e are list[seg[e] .. seg[e + 1])), list [S]
 void psk_moe_plan(hipStream_t st, const int32_t *sel, int S, int experts, int32_t *seg, int32_t *list);
-// x[t] += alpha * sum_i y[t top + i]
-void psk_moe_combine(hipStream_t st, float *x, const float *y, int top, float alpha, int64_t n, int T);
+// x[t] += alpha * sum_i (y[t top + i], or, for a slot whose sel >= n_real (an identity expert), wgt[slot] * h[t]);  y NULL: only the identity slots; sel NULL: only y
+void psk_moe_combine(hipStream_t st, float *x, const float *y, int top, float alpha, int64_t n, int T, const int32_t *sel = nullptr, const float *wgt = nullptr,
+                     int n_real = 0, const float *h = nullptr, int64_t ldh = 0);
 
 // ---- k_latent.hip
 // One token per block.  y[t] = [ dq (q_rank) | ckv (kv_rank) | kr (rot_dim) ]:  cq[t] = rmsnorm(dq) * qnorm;  ring row (pos mod cap):
 // c = rmsnorm(ckv) * kvnorm, kr with its first rot_dims numbers rotated at pos (pairs (i, i + rot_dims/2), angle pos * freq[i]).  Ring at step->state + ring_off: [cap][kv_rank + rot_dim].
 void psk_latent_prep(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int cap, const float *y, int64_t ldy, const float *qnorm, const float *kvnorm,
-                     float eps, int q_rank, int kv_rank, int rot_dim, int rot_dims, const float *freq, int T, float *cq, int64_t ldcq);
+                     float eps, int q_rank, int kv_rank, int rot_dim, int rot_dims, const float *freq, int T, float *cq, int64_t ldcq,
+                     float rot_mag = 1.f); // cos and sin of every rotation of this mixer are multiplied by rot_mag (the same value in all its launches); q_rank 0: no query latent
 // Windowed soft-max attention over expanded keys / values.  q [T][H*(d+dr)] (rotated part not yet rotated), kv [Nw][H*d + H*dv] for the positions
 // first .. first + Nw - 1 where first = max(0, pos0 - window + 1) (the caller expands exactly these ring rows), rotated key parts from the ring.
 void psk_latent_attn(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int cap, const float *q, int64_t ldq, const float *kv, int64_t ldkv,
-                     const float *freq, int H, int d, int dr, int rot_dims, int dv, int kv_rank, int window, float scale, int T, float *o, int64_t ldo);
+                     const float *freq, int H, int d, int dr, int rot_dims, int dv, int kv_rank, int window, float scale, int T, float *o, int64_t ldo,
+                     float rot_mag = 1.f, const float *gate = nullptr, int64_t ldg = 0); // gate [T][H] raw: head h of token t times sigmoid(gate[t][h]) (all forms)
 // The same attention on the matrix cores (fp32 MFMA), 16 tokens of a head per wave; _ok: the sizes it takes (d, dr multiples of 16, dv of 4, dv <= 128).
 bool psk_latent_attn_mfma_ok(int d, int dr, int dv);
 void psk_latent_attn_mfma(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int cap, const float *q, int64_t ldq, const float *kv, int64_t ldkv,
-                          const float *freq, int H, int d, int dr, int rot_dims, int dv, int kv_rank, int window, float scale, int T, float *o, int64_t ldo);
+                          const float *freq, int H, int d, int dr, int rot_dims, int dv, int kv_rank, int window, float scale, int T, float *o, int64_t ldo,
+                          float rot_mag = 1.f, const float *gate = nullptr, int64_t ldg = 0);
 // Single-token step in the absorbed form: nothing is expanded per key, the ring's latents are keys and values for all heads at once.
 // q [H][d + dr] (row stride qstride, rotated part not yet rotated) -> o [H * dv].  ukv: rows uk | uv.  _ok: kv_rank, dr multiples of 16, kv_rank <= 512.
 bool psk_latent_absorbed_ok(int d, int dr, int dv, int R);
 size_t psk_latent_absorbed_scratch(int H, int R, int window);
 void psk_latent_absorbed(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int cap, const float *q, int qstride, const ps_dense *ukv, const float *freq,
-                         int H, int d, int dr, int rot_dims, int dv, int R, int window, float scale, float *scratch, float *o);
+                         int H, int d, int dr, int rot_dims, int dv, int R, int window, float scale, float *scratch, float *o, float rot_mag = 1.f,
+                         const float *gate = nullptr);
 
 // ---- k_winattn.hip
 // y[t] = [ q (H d) | k (G d) | v (G dv) | ... ]: RMS norms over the whole q / k projections (qnorm / knorm, NULL: none), rotation of the first rot_dims numbers of
@@ -141,18 +150,22 @@ void psk_latent_absorbed(hipStream_t st, const ps_seq_step *step, int64_t ring_o
 // step->state + ring_off); then the block means ([block][G d | G dv] at step->state + pool_off, pool > 0) are brought up to date.
 void psk_winattn_prep(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int cap, int64_t pool_off, int pool, const float *y, int64_t ldy, const float *qnorm,
                       const float *knorm, float eps, int H, int G, int d, int dv, int rot_dims, int pairing, const float *freq, int T, float *q, int64_t ldq,
-                      float qt_coef = 0.f, int qt_every = 0); // qt_every > 0: q[t] times 1 + qt_coef ln(floor((pos + 1) / qt_every) + 1)
+                      float qt_coef = 0.f, int qt_every = 0, // qt_every > 0: q[t] times 1 + qt_coef ln(floor((pos + 1) / qt_every) + 1)
+                      int head_norm = 0, // 1: qnorm / knorm are [d] and the norms are taken per head
+                      int v_unit = 0);   // 1: every head's value divided by its own root mean square
 // o[t][h] = gate(t, h) * soft-max attention of q[t][h] over the visible block means and the window's ring rows, scores times scale * temp[h], exp(sink[h]) in the
 // denominator; gate [T][..] raw (sigmoid here; column h, row stride ldg), temp / sink / gate may be NULL.
 void psk_winattn(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int cap, int64_t pool_off, int pool, const float *q, int64_t ldq, const float *gate,
                  int64_t ldg, const float *temp, const float *sink, int H, int G, int d, int dv, int window, float scale, int T, float *o, int64_t ldo,
-                 float softcap = 0.f); // softcap > 0 (all three forms): score <- softcap tanh(score / softcap) behind scale and temperature
+                 float softcap = 0.f, // softcap > 0 (all three forms): score <- softcap tanh(score / softcap) behind scale and temperature
+                 int gate_elem = 0);  // 1 (all three forms): gate [T][H dv], one sigmoid per output element instead of one per head
 // The same attention on the fp32 matrix cores for a portion, 16 tokens of a head per wave; _ok: the sizes it takes (d a multiple of 16, dv of 4, dv <= 128).
 bool psk_winattn_mfma_ok(int d, int dv);
 void psk_winattn_mfma(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int cap, int64_t pool_off, int pool, const float *q, int64_t ldq, const float *gate,
                       int64_t ldg, const float *temp, const float *sink, int H, int G, int d, int dv, int window, float scale, int T, float *o, int64_t ldo,
-                      float softcap = 0.f);
+                      float softcap = 0.f, int gate_elem = 0);
 // A single token on the matrix cores: rows = the heads of a key / value group, the keys spread over waves, partials merged in a second launch (same sizes).
 size_t psk_winattn_step_scratch(int H, int dv, int window, int pool, int64_t max_context);
 void psk_winattn_step(hipStream_t st, const ps_seq_step *step, int64_t ring_off, int cap, int64_t pool_off, int pool, const float *q, const float *gate, const float *temp,
-                      const float *sink, int H, int G, int d, int dv, int window, float scale, int64_t max_context, float *scratch, float *o, float softcap = 0.f);
+                      const float *sink, int H, int G, int d, int dv, int window, float scale, int64_t max_context, float *scratch, float *o, float softcap = 0.f,
+                      int gate_elem = 0);

@@ -12,6 +12,8 @@
 // hand on a weighted average of ALL earlier layers' results instead of its own (depth_mix): the results X_0 .. X_runs of a portion then live side by
 // side (`hist`), a layer's sublayers add into its own X, and the average, the next layer's norms and their group statistics are one launch (psk_front).
 // The feed-forward may be a mixture of experts: the router (fp32) picks per token, the experts' products are grouped launches of the dense kernels.
+// A PRE-NORM layer is  x += mixer(norm1(x)); x += ff(norm2(x)):  no filter, nothing normed behind a sublayer, the second norm reads what the mixer left; its norms
+// (and the final one) may be layer norms (norm_center).
 #include "ps_seq.h"
 
 #include <cmath>
@@ -30,6 +32,7 @@ struct LayerPlan { // one layer RUN (and, as `side`, the second mixer of one)
     int64_t pool_rows = 0; // windowed attention: block means held
     float *freq = nullptr; // rot_dims / 2 angular frequencies (shared by the runs of a layer)
     float act_p = 0.f, act_q = 0.f;
+    float rot_mag = 1.f; // latent: the factor on cos and sin that comes with frequency scaling by wavelength
     int64_t ncat = 0, cqkv = 0;
     // two mixers side by side whose first step is one stacked projection of the same input: the rows of both are ONE matrix (joint, with joint_bias), its
     // result has in_ld columns and this mixer's part starts at column in_off (in_ld == 0: the mixer multiplies by its own in_cat)
@@ -155,25 +158,35 @@ int ps_hip_seq_create(ps_hip_ctx *c, const ps_seq_desc *desc, ps_hip_seq **out) 
             n3 = std::max(n3, H * dv);
             m->weight_bytes += dense_bytes(l.in_cat) + dense_bytes(l.out);
         } else if (l.kind == PS_MIX_LATENT) {
-            if (dv <= 0 || dv > 256 || l.q_rank <= 0 || l.kv_rank <= 0 || l.rot_dim < 0 || l.rot_dims < 0 || l.rot_dims > l.rot_dim || (l.rot_dims & 1) || l.window < 1)
+            if (dv <= 0 || dv > 256 || l.q_rank < 0 || l.kv_rank <= 0 || l.rot_dim < 0 || l.rot_dims < 0 || l.rot_dims > l.rot_dim || (l.rot_dims & 1) || l.window < 0)
                 return at + "latent sizes (vdim <= 256, even rot_dims <= rot_dim)";
-            P.ncat = (int64_t)l.q_rank + l.kv_rank + l.rot_dim;
-            if (!shape(l.in_cat, P.ncat, W) || !shape(l.uq, H * (d + l.rot_dim), l.q_rank) || !shape(l.ukv, H * d + H * dv, l.kv_rank) || !shape(l.out, W, H * dv) ||
-                !l.qnorm || !l.kvnorm)
+            // q_rank 0: the queries come straight from the input, in_cat = q | dkv | gate
+            P.ncat = (l.q_rank > 0 ? (int64_t)l.q_rank : H * (d + l.rot_dim)) + l.kv_rank + l.rot_dim + (l.gated ? H : 0);
+            if (!shape(l.in_cat, P.ncat, W) || (l.q_rank > 0 && !shape(l.uq, H * (d + l.rot_dim), l.q_rank)) || !shape(l.ukv, H * d + H * dv, l.kv_rank) ||
+                !shape(l.out, W, H * dv) || (l.q_rank > 0 && !l.qnorm) || !l.kvnorm || (l.gated && l.gated != 1))
                 return at + "latent tensors";
-            P.cap = (int)(l.window - 1 + B);
+            if (l.yarn_factor != 0.f && (!(l.yarn_factor > 0.f) || l.yarn_original <= 0 || !(l.yarn_fast > 0.f) || !(l.yarn_slow > 0.f) || !(l.rot_base > 1.f)))
+                return at + "latent: frequency scaling constants";
+            if (l.window <= 0 || l.window > m->max_context) m->needs_context = true; // (window 0: everything before the token)
+            const int64_t window = l.window > 0 ? std::min<int64_t>(l.window, m->max_context) : m->max_context;
+            P.d.window = (int32_t)window;
+            P.cap = (int)(window - 1 + B);
+            P.rot_mag = l.yarn_factor > 0.f ? (float)(0.1 * log((double)l.yarn_factor) + 1.0) : 1.f;
             n1 = std::max(n1, P.ncat);
-            nq = std::max(nq, H * (d + l.rot_dim));
-            m->n_t2q = std::max<int64_t>(m->n_t2q, l.q_rank);
+            if (l.q_rank > 0) {
+                nq = std::max(nq, H * (d + l.rot_dim));
+                m->n_t2q = std::max<int64_t>(m->n_t2q, l.q_rank);
+            }
             n3 = std::max(n3, H * dv);
-            nkv = std::max(nkv, (int64_t)(l.window - 1 + B) * (H * d + H * dv));
+            nkv = std::max(nkv, (int64_t)(window - 1 + B) * (H * d + H * dv));
             m->weight_bytes += dense_bytes(l.in_cat) + dense_bytes(l.uq) + dense_bytes(l.ukv) + dense_bytes(l.out);
         } else if (l.kind == PS_MIX_WINATTN) {
             const int64_t G = l.kv_heads;
             if (G <= 0 || H % G || dv <= 0 || dv > 256 || l.rot_dims < 0 || l.rot_dims > d || (l.rot_dims & 1) || l.window < 0 || l.pool < 0)
                 return at + "windowed attention sizes (heads a multiple of kv_heads, vdim <= 256, even rot_dims <= dim)";
             if (l.rot_pairing != PS_ROT_HALVES && l.rot_pairing != PS_ROT_NEIGHBOURS) return at + "rot_pairing";
-            P.ncat = H * d + G * d + G * dv + (l.gated ? H : 0);
+            if (l.gated < 0 || l.gated > 2) return at + "gated: 0 (none), 1 (a row per head) or 2 (a row per output element)";
+            P.ncat = H * d + G * d + G * dv + (l.gated == 2 ? H * dv : l.gated ? H : 0);
             if (!shape(l.in_cat, P.ncat, W) || !shape(l.out, W, H * dv)) return at + "windowed attention tensors";
             if (l.pool > 0 || l.window <= 0 || l.window > m->max_context) m->needs_context = true;
             const int64_t window = l.window > 0 ? std::min<int64_t>(l.window, m->max_context) : m->max_context;
@@ -214,7 +227,9 @@ int ps_hip_seq_create(ps_hip_ctx *c, const ps_seq_desc *desc, ps_hip_seq **out) 
         P.d = desc->layers[P.layer];
         const ps_seq_layer &l = P.d;
         const std::string at = "layer " + std::to_string(P.layer) + ": ";
-        if (l.form != PS_LAYER_SEQUENTIAL && l.form != PS_LAYER_PARALLEL) return fail(at + "unknown layer form");
+        if (l.form != PS_LAYER_SEQUENTIAL && l.form != PS_LAYER_PARALLEL && l.form != PS_LAYER_PRENORM) return fail(at + "unknown layer form");
+        if (l.form == PS_LAYER_PRENORM && (l.canon1 || l.canon2 || l.norm1b || l.norm2b || l.depth_mix)) return fail(at + "a pre-norm layer has no input filter, no norm behind a sublayer and no depth average");
+        if (l.form != PS_LAYER_PRENORM && desc->norm_center) return fail(at + "layer norms (norm_center) are built for pre-norm layers");
         if (!l.norm1 || (l.form == PS_LAYER_SEQUENTIAL && !l.norm1b) || (l.form == PS_LAYER_SEQUENTIAL && !l.canon1)) return fail(at + "norm / canon missing");
         if (l.canon1) { P.off_canon1 = off; off += (int64_t)(desc->canon_taps - 1) * W; }
         if (l.canon1 && (l.norm2 && l.form == PS_LAYER_PARALLEL)) return fail(at + "a parallel layer with an input filter has one norm");
@@ -223,24 +238,32 @@ int ps_hip_seq_create(ps_hip_ctx *c, const ps_seq_desc *desc, ps_hip_seq **out) 
             depth = true;
         }
         if (l.ff_kind != PS_FF_NONE) {
-            if (l.ff_kind != PS_FF_DENSE_XIELU && l.ff_kind != PS_FF_DENSE_SWIGLU && l.ff_kind != PS_FF_MOE_SWIGLU) return fail(at + "unknown feed-forward kind");
-            const bool moe = l.ff_kind == PS_FF_MOE_SWIGLU;
+            if (l.ff_kind != PS_FF_DENSE_XIELU && l.ff_kind != PS_FF_DENSE_SWIGLU && l.ff_kind != PS_FF_MOE_SWIGLU && l.ff_kind != PS_FF_DENSE_RELU_GLU &&
+                l.ff_kind != PS_FF_MOE_RELU2)
+                return fail(at + "unknown feed-forward kind");
+            const bool moe = l.ff_kind == PS_FF_MOE_SWIGLU || l.ff_kind == PS_FF_MOE_RELU2;
+            const int64_t pair = l.ff_kind == PS_FF_MOE_RELU2 ? 1 : 2; // rows of the up matrix per inner unit (a gate and its partner, or one)
             if (moe) {
-                if (l.form != PS_LAYER_PARALLEL || l.canon1) return fail(at + "a mixture of experts needs a parallel layer without an input filter");
-                if (l.experts <= 0 || l.top <= 0 || l.top > l.experts || l.ff <= 0 || !l.router) return fail(at + "mixture-of-experts sizes / router");
-                if (!shape(l.ff_up, (int64_t)l.experts * 2 * l.ff, W) || !shape(l.ff_down, (int64_t)l.experts * W, l.ff)) return fail(at + "expert tensors");
+                if ((l.form != PS_LAYER_PARALLEL && l.form != PS_LAYER_PRENORM) || l.canon1)
+                    return fail(at + "a mixture of experts needs a parallel or pre-norm layer without an input filter");
+                const int rows = l.experts + l.moe_identity; // what the router puts out
+                if (l.experts <= 0 || l.moe_identity < 0 || l.top <= 0 || l.top > rows || l.ff <= 0 || !l.router) return fail(at + "mixture-of-experts sizes / router");
+                if (l.moe_groups > 0 && (rows % l.moe_groups || l.moe_keep <= 0 || l.moe_keep > l.moe_groups || l.top > (int64_t)l.moe_keep * (rows / l.moe_groups)))
+                    return fail(at + "mixture-of-experts groups (equal groups over all router rows, top <= keep * group size)");
+                if (!shape(l.ff_up, (int64_t)l.experts * pair * l.ff, W) || !shape(l.ff_down, (int64_t)l.experts * W, l.ff)) return fail(at + "expert tensors");
                 if (l.shared_up || l.shared_down) {
-                    if (l.shared_ff <= 0 || !shape(l.shared_up, 2 * (int64_t)l.shared_ff, W) || !shape(l.shared_down, W, l.shared_ff)) return fail(at + "shared expert tensors");
+                    if (l.shared_ff <= 0 || !shape(l.shared_up, pair * (int64_t)l.shared_ff, W) || !shape(l.shared_down, W, l.shared_ff)) return fail(at + "shared expert tensors");
                     m->weight_bytes += dense_bytes(l.shared_up) + dense_bytes(l.shared_down);
                 }
                 moe_slots = std::max(moe_slots, B * l.top);
-                moe_experts = std::max<int64_t>(moe_experts, l.experts);
+                moe_experts = std::max<int64_t>(moe_experts, rows);
                 moe_top = std::max<int64_t>(moe_top, l.top);
                 n4 = std::max<int64_t>({n4, (int64_t)l.top * l.ff, (int64_t)l.shared_ff});
-                m->weight_bytes += (dense_bytes(l.ff_up) + dense_bytes(l.ff_down)) / l.experts * l.top + (uint64_t)l.experts * W * 4;
+                m->weight_bytes += (dense_bytes(l.ff_up) + dense_bytes(l.ff_down)) / l.experts * std::min(l.top, l.experts) + (uint64_t)rows * W * 4;
             }
-            const int64_t up_rows = l.ff_kind == PS_FF_DENSE_SWIGLU ? 2 * (int64_t)l.ff : l.ff;
+            const int64_t up_rows = l.ff_kind == PS_FF_DENSE_SWIGLU || l.ff_kind == PS_FF_DENSE_RELU_GLU ? 2 * (int64_t)l.ff : l.ff;
             if (!moe && (!shape(l.ff_up, up_rows, W) || !shape(l.ff_down, W, l.ff))) return fail(at + "feed-forward tensors");
+            if (l.form == PS_LAYER_PRENORM && !l.norm2) return fail(at + "feed-forward norm missing");
             if (l.form == PS_LAYER_SEQUENTIAL) {
                 if (!l.norm2 || !l.norm2b || !l.canon2) return fail(at + "feed-forward norm / canon missing");
                 P.off_canon2 = off; off += (int64_t)(desc->canon_taps - 1) * W;
@@ -294,6 +317,16 @@ int ps_hip_seq_create(ps_hip_ctx *c, const ps_seq_desc *desc, ps_hip_seq **out) 
         const double factor = win && P.d.rot_factor != 0.f ? (double)P.d.rot_factor : 1.0;
         std::vector<float> f(half);
         for (int i = 0; i < half; i++) f[i] = (float)(pow((double)P.d.rot_base, -2.0 * i / (double)P.d.rot_dims) / factor);
+        if (lat && P.d.yarn_factor > 0.f) {
+            // frequency scaling by wavelength: pairs that turn often within the original context keep their frequency, slow ones are divided by the factor, a ramp between
+            const double dims = P.d.rot_dims, base = P.d.rot_base, pi = 3.14159265358979323846;
+            auto turn_index = [&](double turns) { return dims * log((double)P.d.yarn_original / (2.0 * pi * turns)) / (2.0 * log(base)); };
+            const double lo = std::max(floor(turn_index(P.d.yarn_fast)), 0.0), hi = std::min(ceil(turn_index(P.d.yarn_slow)), dims - 1.0);
+            for (int i = 0; i < half; i++) {
+                const double fi = pow(base, -2.0 * i / dims), ramp = std::min(std::max((i - lo) / std::max(hi - lo, 0.001), 0.0), 1.0);
+                f[i] = (float)(fi / (double)P.d.yarn_factor * ramp + fi * (1.0 - ramp));
+            }
+        }
         ok = ok && alloc((void **)&P.freq, half * 4);
         if (ok) ok = hipMemcpyAsync(P.freq, f.data(), half * 4, hipMemcpyHostToDevice, c->stream) == hipSuccess && hipStreamSynchronize(c->stream) == hipSuccess;
         freq_of[P.d.out] = P.freq;
@@ -496,18 +529,19 @@ static void seq_layers(ps_hip_seq *m, float *state, int T, int64_t pos0, bool an
                 psk_dense(st, g);
             }
             psk_winattn_prep(st, m->step, P.off_ring, P.cap, P.off_pool, l.pool, t1, ld1, l.qnorm, l.knorm, D.norm_eps, (int)H, (int)G, (int)d, (int)dv, l.rot_dims,
-                             l.rot_pairing, P.freq, T, m->t2, Hd, l.qtemp_coef, l.qtemp_every);
+                             l.rot_pairing, P.freq, T, m->t2, Hd, l.qtemp_coef, l.qtemp_every, l.head_norm, l.v_unit);
             const float *gate = l.gated ? t1 + Hd + G * d + G * dv : nullptr;
+            const int ge = l.gated == 2; // a gate per output element
             const bool mfma = (m->mode & 2) == 0 && (G * (d + dv)) % 4 == 0 && psk_winattn_mfma_ok((int)d, (int)dv);
             if (mfma && T == 1 && m->win_scratch)
                 psk_winattn_step(st, m->step, P.off_ring, P.cap, P.off_pool, l.pool, m->t2, gate, l.temp, l.sink, (int)H, (int)G, (int)d, (int)dv, l.window, l.scale,
-                                 m->max_context, m->win_scratch, m->t3, l.softcap);
+                                 m->max_context, m->win_scratch, m->t3, l.softcap, ge);
             else if (mfma)
                 psk_winattn_mfma(st, m->step, P.off_ring, P.cap, P.off_pool, l.pool, m->t2, Hd, gate, ld1, l.temp, l.sink, (int)H, (int)G, (int)d, (int)dv, l.window, l.scale,
-                                 T, m->t3, Hv, l.softcap);
+                                 T, m->t3, Hv, l.softcap, ge);
             else
                 psk_winattn(st, m->step, P.off_ring, P.cap, P.off_pool, l.pool, m->t2, Hd, gate, ld1, l.temp, l.sink, (int)H, (int)G, (int)d, (int)dv, l.window, l.scale, T,
-                            m->t3, Hv, l.softcap);
+                            m->t3, Hv, l.softcap, ge);
             out_proj(m->t3, Hv);
         } else if (l.kind == PS_MIX_MINGRU) {
             // t1 = [ z | x | g ] (+ bias); the recurrence and the gate -> t3; out
@@ -519,15 +553,20 @@ static void seq_layers(ps_hip_seq *m, float *state, int T, int64_t pos0, bool an
             psk_mingru_scan(st, m->step, P.off_S, t1, ld1, d, T, m->t3, d);
             out_proj(m->t3, d);
         } else {
+            // t1 = [ dq | dkv ], or with direct queries [ q | dkv | gate ]; the latents' norms, rotation of the shared key part and ring append; attention -> t3; out
             const int64_t dr = l.rot_dim, rs = l.kv_rank + dr, Hv = H * dv, nq = H * (d + dr);
-            float *cq = m->t2, *q = m->t2 + (int64_t)D.max_batch * m->n_t2q;
+            const bool direct = l.q_rank == 0;
+            float *cq = m->t2, *q = direct ? m->t1 : m->t2 + (int64_t)D.max_batch * m->n_t2q;
+            const int64_t ldq = direct ? P.ncat : nq;
+            const float *gate = l.gated ? m->t1 + P.ncat - H : nullptr;
             psk_dense(st, mm(l.in_cat, m->h, W, m->t1, P.ncat));
-            psk_latent_prep(st, m->step, P.off_ring, P.cap, m->t1, P.ncat, l.qnorm, l.kvnorm, D.norm_eps, l.q_rank, l.kv_rank, (int)dr, l.rot_dims, P.freq, T, cq, l.q_rank);
-            psk_dense(st, mm(l.uq, cq, l.q_rank, q, nq));
+            psk_latent_prep(st, m->step, P.off_ring, P.cap, direct ? m->t1 + nq : m->t1, P.ncat, l.qnorm, l.kvnorm, D.norm_eps, l.q_rank, l.kv_rank, (int)dr, l.rot_dims, P.freq, T,
+                            cq, l.q_rank, P.rot_mag);
+            if (!direct) psk_dense(st, mm(l.uq, cq, l.q_rank, q, nq));
             const bool plain = (m->mode & 2) != 0, rows4 = (l.kv_rank + dr) % 4 == 0 && l.kv_rank % 4 == 0;
             if (T == 1 && !plain && m->abs_scratch && psk_latent_absorbed_ok((int)d, (int)dr, (int)dv, l.kv_rank)) {
                 psk_latent_absorbed(st, m->step, P.off_ring, P.cap, q, (int)(d + dr), l.ukv, P.freq, (int)H, (int)d, (int)dr, l.rot_dims, (int)dv, l.kv_rank, l.window,
-                                    l.scale, m->abs_scratch, m->t3);
+                                    l.scale, m->abs_scratch, m->t3, P.rot_mag, gate);
             } else {
                 // the window's keys and values, expanded from the ring rows  max(0, pos0 - window + 1) .. pos0 + T - 1
                 auto g = mm(l.ukv, state + P.off_ring, rs, m->kvx, H * d + Hv);
@@ -535,11 +574,11 @@ static void seq_layers(ps_hip_seq *m, float *state, int T, int64_t pos0, bool an
                 g.T = any_pos ? l.window - 1 + T : (int)(std::min<int64_t>(pos0, l.window - 1) + T);
                 psk_dense(st, g);
                 if (!plain && rows4 && psk_latent_attn_mfma_ok((int)d, (int)dr, (int)dv))
-                    psk_latent_attn_mfma(st, m->step, P.off_ring, P.cap, q, nq, m->kvx, H * d + Hv, P.freq, (int)H, (int)d, (int)dr, l.rot_dims, (int)dv, l.kv_rank, l.window,
-                                         l.scale, T, m->t3, Hv);
+                    psk_latent_attn_mfma(st, m->step, P.off_ring, P.cap, q, ldq, m->kvx, H * d + Hv, P.freq, (int)H, (int)d, (int)dr, l.rot_dims, (int)dv, l.kv_rank, l.window,
+                                         l.scale, T, m->t3, Hv, P.rot_mag, gate, P.ncat);
                 else
-                    psk_latent_attn(st, m->step, P.off_ring, P.cap, q, nq, m->kvx, H * d + Hv, P.freq, (int)H, (int)d, (int)dr, l.rot_dims, (int)dv, l.kv_rank, l.window,
-                                    l.scale, T, m->t3, Hv);
+                    psk_latent_attn(st, m->step, P.off_ring, P.cap, q, ldq, m->kvx, H * d + Hv, P.freq, (int)H, (int)d, (int)dr, l.rot_dims, (int)dv, l.kv_rank, l.window,
+                                    l.scale, T, m->t3, Hv, P.rot_mag, gate, P.ncat);
             }
             out_proj(m->t3, Hv);
         }
@@ -554,34 +593,45 @@ static void seq_layers(ps_hip_seq *m, float *state, int T, int64_t pos0, bool an
         const ps_seq_layer &l = P.d;
         auto g = mm(l.ff_up, in, W, m->t4, l.ff);
         if (l.ff_kind == PS_FF_DENSE_SWIGLU) g.act = PSD_ACT_SILU_PAIR;
+        else if (l.ff_kind == PS_FF_DENSE_RELU_GLU) g.act = PSD_ACT_RELU_PAIR;
         else { g.act = PSD_ACT_XIELU; g.act_p = P.act_p; g.act_q = P.act_q; }
+        if (l.ff_kind != PS_FF_DENSE_XIELU) g.bias = l.ff_up_bias;
         psk_dense(st, g);
     };
-    // The feed-forward of a parallel layer on `in`, added to xr times alpha.  Mixture of experts: slot s = t top + i is token t's i-th expert; the router's
-    // score scales what the expert READS (the A operand of its first product), a few tokens run grouped mat-vecs, a portion tiles over the slots sorted by expert.
+    // The feed-forward of a parallel or pre-norm layer on `in`, added to xr times alpha.  Mixture of experts: slot s = t top + i is token t's i-th choice; the router's
+    // score scales what the expert READS (the A operand of its first product) or, moe_weight_output, what it puts out (the rows of its inner activation: the second
+    // product is linear); a few tokens run grouped mat-vecs, a portion tiles over the slots sorted by expert.  A choice beyond the experts that have matrices is an
+    // identity expert: no product touches its slot, and its weight times the input joins the sum.
     auto feed_forward = [&](const LayerPlan &P, const float *in, float *xr, float alpha) {
         const ps_seq_layer &l = P.d;
-        if (l.ff_kind != PS_FF_MOE_SWIGLU) {
+        const bool moe = l.ff_kind == PS_FF_MOE_SWIGLU || l.ff_kind == PS_FF_MOE_RELU2;
+        if (!moe) {
             ff_up(P, in);
             auto g = mm(l.ff_down, m->t4, l.ff, xr, W);
             g.accum = 1; g.alpha = alpha;
+            if (l.ff_kind != PS_FF_DENSE_XIELU) g.bias = l.ff_down_bias;
             psk_dense(st, g);
             return;
         }
-        const int E = l.experts, top = l.top, S = T * top;
-        psk_moe_route(st, in, W, l.router, l.shared_gate, E, top, l.moe_norm_top, W, T, m->moe_sel, m->moe_wgt, m->moe_sg);
+        const int E = l.experts, rows = E + l.moe_identity, top = l.top, S = T * top;
+        const int act = l.ff_kind == PS_FF_MOE_RELU2 ? PSD_ACT_RELU2 : PSD_ACT_SILU_PAIR;
+        psk_moe_route(st, in, W, l.router, l.shared_gate, rows, top, l.moe_norm_top, W, T, m->moe_sel, m->moe_wgt, m->moe_sg, l.moe_softmax, l.moe_correction, l.moe_groups,
+                      l.moe_keep);
         const bool mv = !tiled && T <= 8 && (size_t)std::max<int64_t>(W, (int64_t)top * l.ff) * 4 + 64 <= 128 * 1024;
-        if (!mv) psk_moe_plan(st, m->moe_sel, S, E, m->moe_seg, m->moe_list);
+        if (!mv) psk_moe_plan(st, m->moe_sel, S, rows, m->moe_seg, m->moe_list);
         auto grouped = [&](psk_dense_args &g) {
             g.groups = E; g.g_sel = m->moe_sel;
             if (!mv) { g.g_seg = m->moe_seg; g.g_list = m->moe_list; }
         };
         {
             auto g = mm(l.ff_up, in, W, m->t4, l.ff);
-            g.act = PSD_ACT_SILU_PAIR; g.T = S; g.g_adiv = top; g.g_scale = m->moe_wgt;
+            g.act = act; g.T = S; g.g_adiv = top;
+            if (l.moe_weight_output) g.out_scale = m->moe_wgt; // (a row of the result is a slot)
+            else g.g_scale = m->moe_wgt;
             grouped(g);
             psk_dense(st, g);
         }
+        bool summed = false; // the identity slots' share has joined the stream
         {
             auto g = mm(l.ff_down, m->t4, l.ff, xr, W);
             grouped(g);
@@ -589,11 +639,15 @@ static void seq_layers(ps_hip_seq *m, float *state, int T, int64_t pos0, bool an
             else if (top == 1) { g.T = S; g.accum = 1; g.alpha = alpha; }
             else { g.T = S; g.out = m->moe_y; } // (two slots of a token sit in different tiles: per-slot results, summed below)
             psk_dense(st, g);
-            if (!mv && top > 1) psk_moe_combine(st, xr, m->moe_y, top, alpha, W, T);
+            if (!mv && top > 1) {
+                psk_moe_combine(st, xr, m->moe_y, top, alpha, W, T, l.moe_identity ? m->moe_sel : nullptr, m->moe_wgt, E, in, W);
+                summed = true;
+            }
         }
+        if (l.moe_identity && !summed) psk_moe_combine(st, xr, nullptr, top, alpha, W, T, m->moe_sel, m->moe_wgt, E, in, W);
         if (l.shared_up) {
             auto g = mm(l.shared_up, in, W, m->t4, l.shared_ff);
-            g.act = PSD_ACT_SILU_PAIR;
+            g.act = act;
             psk_dense(st, g);
             auto g2 = mm(l.shared_down, m->t4, l.shared_ff, xr, W);
             g2.accum = 1; g2.alpha = alpha; g2.out_scale = l.shared_gate ? m->moe_sg : nullptr;
@@ -607,7 +661,17 @@ static void seq_layers(ps_hip_seq *m, float *state, int T, int64_t pos0, bool an
         const ps_seq_layer &l = P.d;
         const LayerPlan *next = li + 1 < n_runs ? &m->L[li + 1] : nullptr;
         const float res = l.res_scale != 0.f ? l.res_scale : 1.f;
-        if (l.form == PS_LAYER_PARALLEL && !l.canon1) {
+        if (l.form == PS_LAYER_PRENORM) {
+            // x += mixer(norm1(x)), then x += ff(norm2(x)): each sublayer's front is one launch, its output projection adds straight into the residual stream
+            psk_front(st, m->x, 0, 1, nullptr, nullptr, nullptr, l.norm1, m->h, nullptr, nullptr, m->groups, D.norm_offset, D.norm_eps, W, T, D.norm_center);
+            joint_in(P);
+            mixer(P, m->x, l.mix_scale);
+            if (P.side) mixer(*P.side, m->x, P.side->d.mix_scale);
+            if (l.ff_kind != PS_FF_NONE) {
+                psk_front(st, m->x, 0, 1, nullptr, nullptr, nullptr, l.norm2, m->h, nullptr, nullptr, m->groups, D.norm_offset, D.norm_eps, W, T, D.norm_center);
+                feed_forward(P, m->h, m->x, 1.f);
+            }
+        } else if (l.form == PS_LAYER_PARALLEL && !l.canon1) {
             // No input filter: one launch makes the layer's input (with depth_mix: the previous layer's average over X_0 .. X_li, kept as this layer's X to add
             // into) and both sublayers' norms; mixers and feed-forward add their output projections, times res, straight into the layer's X
             float *xr = m->hist ? m->hist + (int64_t)(li + 1) * BW : m->x;
@@ -657,6 +721,8 @@ static void seq_head(ps_hip_seq *m, const int32_t *idx, int rows) {
         const int runs = (int)m->L.size();
         psk_front(st, m->hist, (int64_t)D.max_batch * D.width, runs + 1, m->L[runs - 1].d.depth_mix, idx, nullptr, D.final_norm, m->xn, nullptr, nullptr, m->groups,
                   D.norm_offset, D.norm_eps, D.width, rows);
+    } else if (D.norm_center) {
+        psk_front(st, m->x, 0, 1, nullptr, idx, nullptr, D.final_norm, m->xn, nullptr, nullptr, m->groups, D.norm_offset, D.norm_eps, D.width, rows, 1);
     } else {
         psk_rmsnorm(st, m->x, D.width, idx, D.final_norm, D.norm_offset, D.norm_eps, D.width, rows, m->xn, D.width, m->groups);
     }
@@ -767,19 +833,25 @@ int ps_hip_seq_bench_kernel(ps_hip_seq *m, int which, int T, int reps, double *u
     std::vector<psk_dense_args> launches; // one per layer that has the matrix: every launch streams its own (cold) weights, as in a step
     double per_bytes = 0, per_flops = 0;
     for (const LayerPlan &P : m->L) {
-        if (P.d.ff_kind == PS_FF_NONE || (P.d.ff_kind == PS_FF_MOE_SWIGLU) != moe) continue;
+        const bool is_moe = P.d.ff_kind == PS_FF_MOE_SWIGLU || P.d.ff_kind == PS_FF_MOE_RELU2;
+        if (P.d.ff_kind == PS_FF_NONE || is_moe != moe) continue;
         psk_dense_args g;
         g.T = T; g.pack = m->pack; g.pack_bytes = m->pack_bytes;
         if (moe) {
             // the routing of this layer (all layers' launches below then reuse the LAST layer's routing: the same shapes and spread)
             const int top = P.d.top, S = T * top;
             const bool mv = T <= 8;
-            psk_moe_route(c->stream, m->h, W, P.d.router, P.d.shared_gate, P.d.experts, top, P.d.moe_norm_top, W, T, m->moe_sel, m->moe_wgt, m->moe_sg);
-            if (!mv) psk_moe_plan(c->stream, m->moe_sel, S, P.d.experts, m->moe_seg, m->moe_list);
+            const int rows = P.d.experts + P.d.moe_identity;
+            psk_moe_route(c->stream, m->h, W, P.d.router, P.d.shared_gate, rows, top, P.d.moe_norm_top, W, T, m->moe_sel, m->moe_wgt, m->moe_sg, P.d.moe_softmax,
+                          P.d.moe_correction, P.d.moe_groups, P.d.moe_keep);
+            if (!mv) psk_moe_plan(c->stream, m->moe_sel, S, rows, m->moe_seg, m->moe_list);
             g.groups = P.d.experts; g.g_sel = m->moe_sel;
             if (!mv) { g.g_seg = m->moe_seg; g.g_list = m->moe_list; }
             if (which == 2) {
-                g.w = P.d.ff_up; g.a = m->h; g.lda = W; g.out = m->t4; g.ldo = P.d.ff; g.act = PSD_ACT_SILU_PAIR; g.T = S; g.g_adiv = top; g.g_scale = m->moe_wgt;
+                g.w = P.d.ff_up; g.a = m->h; g.lda = W; g.out = m->t4; g.ldo = P.d.ff; g.T = S; g.g_adiv = top;
+                g.act = P.d.ff_kind == PS_FF_MOE_RELU2 ? PSD_ACT_RELU2 : PSD_ACT_SILU_PAIR;
+                if (P.d.moe_weight_output) g.out_scale = m->moe_wgt;
+                else g.g_scale = m->moe_wgt;
             } else {
                 g.w = P.d.ff_down; g.a = m->t4; g.lda = P.d.ff; g.ldo = W;
                 if (mv) { g.T = T; g.g_inner = top; g.out = m->y; }
@@ -791,6 +863,7 @@ int ps_hip_seq_bench_kernel(ps_hip_seq *m, int which, int T, int reps, double *u
         } else if (which == 0) {
             g.w = P.d.ff_up; g.a = m->h; g.lda = m->d.width; g.out = m->t4; g.ldo = P.d.ff;
             if (P.d.ff_kind == PS_FF_DENSE_SWIGLU) g.act = PSD_ACT_SILU_PAIR;
+            else if (P.d.ff_kind == PS_FF_DENSE_RELU_GLU) { g.act = PSD_ACT_RELU_PAIR; g.bias = P.d.ff_up_bias; }
             else { g.act = PSD_ACT_XIELU; g.act_p = P.act_p; g.act_q = P.act_q; }
         }
         else { g.w = P.d.ff_down; g.a = m->t4; g.lda = P.d.ff; g.out = m->y; g.ldo = m->d.width; }

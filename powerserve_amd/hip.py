@@ -99,7 +99,10 @@ SeqLayer._fields_ = ([(n, C.c_int32) for n in ("kind", "heads", "kv_heads", "dim
                 [(n, C.c_void_p) for n in ("in_bias", "knorm", "temp", "sink")] + [("tau", C.c_float)] +
                 [("res_scale", C.c_float), ("depth_mix", C.c_void_p), ("softcap", C.c_float), ("qtemp_coef", C.c_float), ("qtemp_every", C.c_int32)] +
                 [(n, C.c_int32) for n in ("experts", "top", "shared_ff", "moe_norm_top")] +
-                [(n, C.c_void_p) for n in ("router", "shared_gate", "shared_up", "shared_down")])
+                [(n, C.c_void_p) for n in ("router", "shared_gate", "shared_up", "shared_down")] +
+                [("head_norm", C.c_int32), ("v_unit", C.c_int32), ("yarn_factor", C.c_float), ("yarn_fast", C.c_float), ("yarn_slow", C.c_float), ("yarn_original", C.c_int32)] +
+                [("ff_up_bias", C.c_void_p), ("ff_down_bias", C.c_void_p)] +
+                [(n, C.c_int32) for n in ("moe_identity", "moe_softmax", "moe_groups", "moe_keep", "moe_weight_output")] + [("moe_correction", C.c_void_p)])
 
 
 class SeqDesc(C.Structure):
@@ -107,7 +110,7 @@ class SeqDesc(C.Structure):
     _fields_ = ([(n, C.c_int32) for n in ("n_layers", "width", "vocab", "canon_taps", "max_batch", "n_slots", "compute")] +
                 [("norm_eps", C.c_float), ("norm_offset", C.c_float), ("logit_scale", C.c_float)] +
                 [("embed", C.c_void_p), ("head", C.c_void_p), ("final_norm", C.c_void_p), ("layers", C.POINTER(SeqLayer))] +
-                [("embed_scale", C.c_float)] + [(n, C.c_int32) for n in ("loop_start", "loop_stop", "loop_times", "max_context", "norm_groups")])
+                [("embed_scale", C.c_float)] + [(n, C.c_int32) for n in ("loop_start", "loop_stop", "loop_times", "max_context", "norm_groups", "norm_center")])
 
 
 _LIB = None

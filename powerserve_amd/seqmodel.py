@@ -26,6 +26,16 @@ the vector, no input filter, a scaled embedding; what a layer hands on is a weig
                     output W_o (S * silu(W_g h))
 Feed-forward: SiLU-gated dense, or a mixture of such experts -- sigmoid router in fp32, the 'top' largest scores, a chosen expert's score multiplies its INPUT,
 plus a shared expert for every token times sigmoid of a one-row projection.
+
+Pokatar: PRE-NORM layers,  x += mix(ln1(x)); x += mlp(ln2(x)), the norms layer norms (mean taken off, a weight, no bias), logits against the embedding table itself.
+Mixers:
+  attention         grouped-query causal soft-max attention without positions: per-head RMS norms of q and k (one weight vector shared by the heads), every head's
+                    value a unit-rms vector, a sink of score 0 in the denominator, sigmoid(W_g h) element by element on the concatenated heads
+  latent_attention  queries straight from the input, keys / values through one normed latent plus one rotated key part shared by the heads; rotate-half rotary whose
+                    frequencies are scaled by wavelength (slow pairs divided by a factor, a ramp between, cos and sin stretched); causal; a sigmoid gate per head
+Feed-forward: relu-gated dense with biases, or a mixture of squared-relu experts -- soft-max router in fp32 over experts AND identity experts (output = input), a
+correction added to the scores for the choice only, the choice limited to the best groups of neighbouring router rows, the chosen scores (not renormalised) on the
+experts' outputs, plus a shared expert for every token.
 """
 from __future__ import annotations
 
@@ -39,8 +49,8 @@ from . import hip
 from .safetensors_io import SafeTensors
 
 MIX_WKV, MIX_DELTA, MIX_LATENT, MIX_WINATTN, MIX_GLA, MIX_MINGRU = 1, 2, 3, 4, 5, 6
-FF_NONE, FF_DENSE_XIELU, FF_DENSE_SWIGLU, FF_MOE_SWIGLU = 0, 1, 2, 3
-LAYER_SEQUENTIAL, LAYER_PARALLEL = 0, 1
+FF_NONE, FF_DENSE_XIELU, FF_DENSE_SWIGLU, FF_MOE_SWIGLU, FF_DENSE_RELU_GLU, FF_MOE_RELU2 = 0, 1, 2, 3, 4, 5
+LAYER_SEQUENTIAL, LAYER_PARALLEL, LAYER_PRENORM = 0, 1, 2
 ROT_HALVES, ROT_NEIGHBOURS = 0, 1
 
 
@@ -240,6 +250,122 @@ def _zusolix_layers(cfg: dict, st: SafeTensors, up) -> tuple[list, dict]:
     return layers, top
 
 
+def sink_attention_mixer(L, st: SafeTensors, up, m: str, mc: dict, where: str):
+    """Fill descriptor L with grouped-query causal attention whose q / k norms are taken per head (one weight vector of `dim`), whose values are unit-rms
+    vectors, whose soft-max has a sink of score 0, and whose gate has a row per output element: MIX_WINATTN with those switches on.  What the file does not
+    have does not exist (no norm, no gate)."""
+    L.kind = MIX_WINATTN
+    L.heads, L.dim = int(mc["heads"]), int(mc["dim"])
+    L.kv_heads, L.vdim = int(mc.get("kv_heads") or L.heads), int(mc.get("vdim") or L.dim)
+    if L.heads % L.kv_heads:
+        raise ConfigError(f"{where}: {L.heads} heads over {L.kv_heads} key / value heads")
+    L.window, L.pool, L.rot_dims, L.rot_base, L.rot_pairing = int((mc.get("mask") or {}).get("size") or 0), 0, 0, 10000.0, ROT_HALVES
+    L.scale = float(mc["scale"]) if mc.get("scale") is not None else L.dim ** -0.5
+    L.head_norm, L.v_unit = 1, 1
+    rows = [(m + "q", L.heads * L.dim), (m + "k", L.kv_heads * L.dim), (m + "v", L.kv_heads * L.vdim)]
+    if m + "g" in st:
+        L.gated = 2
+        rows.append((m + "g", L.heads * L.vdim))
+    for n, r in rows:
+        if st.shape(n)[0] != r:
+            raise ConfigError(f"tensor {n}: {st.shape(n)[0]} rows, the configuration gives {r}")
+    L.in_cat = up.mat(_stack(st, [n for n, _ in rows]))
+    if m + "q.norm" in st:
+        L.qnorm = up.vec(_expect(st, m + "q.norm", (L.dim,)))
+    if m + "k.norm" in st:
+        L.knorm = up.vec(_expect(st, m + "k.norm", (L.dim,)))
+    L.sink = up.vec(np.zeros(L.heads, np.float32))  # exp(0) = 1 joins every head's denominator
+    L.out = up.mat(st.bf16_bits(m + "o"))
+
+
+def shared_key_latent_mixer(L, st: SafeTensors, up, m: str, mc: dict, where: str):
+    """Fill descriptor L with latent attention whose queries come straight from the input (MIX_LATENT with q_rank 0): q | dkv | g stacked, uk | uv stacked,
+    causal (window 0) unless the configuration has a mask, frequency scaling from rot.scaling, a gate row per head where the file has one."""
+    L.kind, L.q_rank = MIX_LATENT, 0
+    L.heads, L.dim, L.vdim = int(mc["heads"]), int(mc["dim"]), int(mc.get("vdim") or mc["dim"])
+    L.kv_rank, L.rot_dim = int(mc["kv_rank"]), int(mc["rot_dim"])
+    rot = mc.get("rot") or {}
+    L.rot_dims, L.rot_base = int(rot.get("dims") or 0), float(rot.get("base") or 10000.0)
+    sc = rot.get("scaling") or {}
+    if sc:
+        L.yarn_factor, L.yarn_fast, L.yarn_slow, L.yarn_original = float(sc["factor"]), float(sc["fast"]), float(sc["slow"]), int(sc["original"])
+    L.window, L.scale = int((mc.get("mask") or {}).get("size") or 0), float(mc["scale"])
+    rows = [(m + "q", L.heads * (L.dim + L.rot_dim)), (m + "dkv", L.kv_rank + L.rot_dim)]
+    if m + "g" in st:
+        L.gated = 1
+        rows.append((m + "g", L.heads))
+    for n, r in rows + [(m + "uk", L.heads * L.dim), (m + "uv", L.heads * L.vdim)]:
+        if st.shape(n)[0] != r:
+            raise ConfigError(f"tensor {n}: {st.shape(n)[0]} rows, the configuration gives {r} ({where})")
+    L.in_cat = up.mat(_stack(st, [n for n, _ in rows]))
+    L.ukv = up.mat(_stack(st, [m + "uk", m + "uv"]))
+    L.kvnorm = up.vec(_expect(st, m + "dkv.norm", (L.kv_rank,)))
+    L.out = up.mat(st.bf16_bits(m + "o"))
+
+
+def relu_feed_forward(L, st: SafeTensors, up, p: str, mlp: dict, width: int, where: str):
+    """Fill descriptor L's feed-forward: 'dense' = relu-gated with optional biases (gate / up rows and their biases interleaved), 'moe' = squared-relu experts
+    e0, e1, ... stacked into one matrix each way, an fp32 router over experts + identity experts with an optional correction and group limit, the scores on the
+    experts' outputs, an optional shared expert."""
+    kind = mlp.get("kind")
+    if kind == "dense":
+        L.ff_kind, L.ff = FF_DENSE_RELU_GLU, int(mlp["ff"])
+        L.ff_up, L.ff_down = up.mat(_gate_up(st, p, L.ff, width, where)), up.mat(st.bf16_bits(p + "down"))
+        if p + "gate.b" in st or p + "up.b" in st:
+            b = [_expect(st, p + n + ".b", (L.ff,)) if p + n + ".b" in st else np.zeros(L.ff, np.float32) for n in ("gate", "up")]
+            L.ff_up_bias = up.vec(np.stack(b, axis=1).reshape(-1))
+        if p + "down.b" in st:
+            L.ff_down_bias = up.vec(_expect(st, p + "down.b", (width,)))
+    elif kind == "moe":
+        r = mlp["router"]
+        L.ff_kind, L.ff, L.experts, L.top = FF_MOE_RELU2, int(mlp["expert"]["ff"]), int(r["experts"]), int(r["top"])
+        L.moe_identity, L.moe_softmax, L.moe_weight_output = int(r.get("identity") or 0), 1, 1
+        rows = L.experts + L.moe_identity
+        gr = r.get("groups") or {}
+        L.moe_groups, L.moe_keep = int(gr.get("count") or 0), int(gr.get("keep") or 0)
+        if not 0 < L.top <= rows or (L.moe_groups and (rows % L.moe_groups or not 0 < L.moe_keep <= L.moe_groups or L.top > L.moe_keep * (rows // L.moe_groups))):
+            raise ConfigError(f"{where}: top {L.top} of {rows} router rows in {L.moe_groups} groups of which {L.moe_keep} stay")
+        for e in range(L.experts):
+            if st.shape(f"{p}e{e}.up") != (L.ff, width) or st.shape(f"{p}e{e}.down") != (width, L.ff):
+                raise ConfigError(f"{where}: expert {e} shapes {st.shape(f'{p}e{e}.up')} / {st.shape(f'{p}e{e}.down')}, the configuration gives {(L.ff, width)}")
+        L.ff_up = up.mat(_stack(st, [f"{p}e{e}.up" for e in range(L.experts)]))
+        L.ff_down = up.mat(_stack(st, [f"{p}e{e}.down" for e in range(L.experts)]))
+        L.router = up.vec(_expect(st, p + "router", (rows, width)))
+        if p + "correction" in st:
+            L.moe_correction = up.vec(_expect(st, p + "correction", (rows,)))
+        if mlp.get("shared"):
+            L.shared_ff = int(mlp["shared"]["ff"])
+            if st.shape(p + "shared.up") != (L.shared_ff, width) or st.shape(p + "shared.down") != (width, L.shared_ff):
+                raise ConfigError(f"{where}: shared expert shapes, the configuration gives {(L.shared_ff, width)}")
+            L.shared_up, L.shared_down = up.mat(st.bf16_bits(p + "shared.up")), up.mat(st.bf16_bits(p + "shared.down"))
+    else:
+        raise ConfigError(f"{where}: feed-forward kind {kind!r} is not known")
+
+
+def _pokatar_layers(cfg: dict, st: SafeTensors, up) -> tuple[list, dict]:
+    width = int(cfg["width"])
+    layers = []
+    for i, lc in enumerate(cfg["layers"]):
+        p, mc, kind = f"l{i}.", lc["mixer"], lc["type"]
+        L = hip.SeqLayer()
+        L.form, L.mix_scale = LAYER_PRENORM, 1.0
+        L.norm1 = up.vec(_expect(st, p + "norm1", (width,)))
+        if kind == "attention":
+            sink_attention_mixer(L, st, up, p + "mix.", mc, f"layer {i}")
+        elif kind == "latent_attention":
+            shared_key_latent_mixer(L, st, up, p + "mix.", mc, f"layer {i}")
+        else:
+            raise ConfigError(f"layer {i}: mixer type {kind!r} is not known")
+        if lc.get("mlp"):
+            L.norm2 = up.vec(_expect(st, p + "norm2", (width,)))
+            relu_feed_forward(L, st, up, p + "mlp.", lc["mlp"], width, f"layer {i}")
+        layers.append(L)
+    embed = up.mat(st.bf16_bits("embed"))
+    top = dict(width=width, vocab=int(cfg["vocab"]), canon_taps=1, norm_eps=float(cfg["norm"]["eps"]), norm_offset=0.0, norm_center=1, logit_scale=1.0,
+               embed=embed, head=embed, final_norm=up.vec(_expect(st, "final.norm", (width,))))
+    return layers, top
+
+
 def _vobisun_layers(cfg: dict, st: SafeTensors, up) -> tuple[list, dict]:
     width = int(cfg["width"])
     taps = int((cfg.get("canon") or {}).get("taps") or 1)
@@ -279,7 +405,7 @@ def _vobisun_layers(cfg: dict, st: SafeTensors, up) -> tuple[list, dict]:
     return layers, top
 
 
-ARCHITECTURES = {"Ranutar": _ranutar_layers, "Vobisun": _vobisun_layers, "Zusolix": _zusolix_layers}
+ARCHITECTURES = {"Ranutar": _ranutar_layers, "Vobisun": _vobisun_layers, "Zusolix": _zusolix_layers, "Pokatar": _pokatar_layers}
 
 
 def read_config(model_dir: str) -> dict:

@@ -406,3 +406,174 @@ def run_zusolix(cfg, W, tokens, per_layer=None, use_depth=True, attn_kw=None, gr
         if per_layer is not None:
             per_layer.append(x)
     return grouped_norm(x, W["final.norm"], groups, eps) @ W["head"].T
+
+
+# ------------------------------------------------------------------------------------------------ Pokatar
+# Sequential pre-norm layers,  x += mixer(ln1(x)); x += ff(ln2(x)),  with mean-centred layer norms (a weight, no bias), two kinds of causal
+# attention (grouped-query with per-head q / k norms, unit-rms values, a zero-score sink and an element-wise output gate; latent attention with a
+# direct query projection, YaRN-scaled rotate-half rotary on a shared key part and a per-head output gate), a relu-gated dense feed-forward with
+# biases, and a mixture of squared-relu experts behind a soft-max router with a selection correction, group-limited choice and identity experts.
+# The logits are the final layer norm against the embedding table itself.
+
+
+def centred_norm(a, w, eps):
+    """(a - mean) / sqrt(var + eps) * w, var the mean of the squared deviations."""
+    dev = a - np.mean(a, axis=-1, keepdims=True)
+    return dev / np.sqrt(np.mean(dev * dev, axis=-1, keepdims=True) + eps) * w
+
+
+def sink_softmax(scores, use_sink=True):
+    """exp(s_j) / (1 + sum exp(s)): one more term of score 0 that carries no value."""
+    m = max(np.max(scores), 0.0) if use_sink else np.max(scores)
+    e = np.exp(scores - m)
+    return e / (e.sum() + (np.exp(-m) if use_sink else 0.0))
+
+
+def sink_gated_attention(W, pre, h, mc, eps, reach=None, use_sink=True, norm_values=True, gate_per_element=True):
+    """Grouped-query causal attention: per-head RMS norms of q and k (one weight vector of `dim` shared by the heads), values divided by their
+    own root mean square, no positions, the sink soft-max, sigmoid(W_g h) element by element on the concatenated heads."""
+    T = h.shape[0]
+    H, G, d, dv = mc["heads"], mc["kv_heads"], mc["dim"], mc["vdim"]
+    q = (h @ W[pre + "q"].T).reshape(T, H, d)
+    k = (h @ W[pre + "k"].T).reshape(T, G, d)
+    v = (h @ W[pre + "v"].T).reshape(T, G, dv)
+    q = unit_rms(q, eps) * W[pre + "q.norm"]
+    k = unit_rms(k, eps) * W[pre + "k.norm"]
+    if norm_values:
+        v = unit_rms(v, eps)
+    gate = sigmoid(h @ W[pre + "g"].T)
+    out = np.zeros((T, H, dv))
+    for i in range(T):
+        lo = 0 if reach is None else max(0, i - reach + 1)
+        for hd in range(H):
+            g = hd // (H // G)
+            s = np.array([q[i, hd] @ k[j, g] for j in range(lo, i + 1)]) * mc["scale"]
+            p = sink_softmax(s, use_sink)
+            out[i, hd] = p @ v[lo:i + 1, g]
+    out = out.reshape(T, H * dv)
+    out = out * gate if gate_per_element else out
+    return out @ W[pre + "o"].T
+
+
+def yarn_frequencies(rot):
+    """f_i = base^(-2i/dims) blended with f_i / factor by a ramp over the pair index; -> (frequencies, the factor on cos and sin)."""
+    dims, base, sc = rot["dims"], rot["base"], rot.get("scaling")
+    f = np.array([base ** (-2.0 * i / dims) for i in range(dims // 2)])
+    if not sc:
+        return f, 1.0
+    def turn_index(t):
+        return dims * np.log(sc["original"] / (2.0 * np.pi * t)) / (2.0 * np.log(base))
+    lo = max(np.floor(turn_index(sc["fast"])), 0)
+    hi = min(np.ceil(turn_index(sc["slow"])), dims - 1)
+    ramp = np.clip((np.arange(dims // 2) - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+    return f / sc["factor"] * ramp + f * (1.0 - ramp), 0.1 * np.log(sc["factor"]) + 1.0
+
+
+def rotate_halves(vec, pos, freqs, mag):
+    """Pairs (i, i + n) of the first 2n numbers, n = len(freqs), turned by pos * freqs[i]; cos and sin both times mag."""
+    n = len(freqs)
+    out = np.array(vec, dtype=np.float64)
+    a = pos * freqs
+    c, s = np.cos(a) * mag, np.sin(a) * mag
+    u, v = vec[..., :n], vec[..., n:2 * n]
+    out[..., :n] = u * c - v * s
+    out[..., n:2 * n] = v * c + u * s
+    return out
+
+
+def shared_key_latent_attention(W, pre, h, mc, eps, reach=None, use_scaling=True, use_gate=True):
+    """q straight from the input, laid out per head as [dim plain | rot_dim rotated]; keys and values from one normed latent per token plus one
+    rotated key part shared by the heads; ordinary soft-max; each head's output times sigmoid of its row of W_g."""
+    T = h.shape[0]
+    H, d, dr, dv, R = mc["heads"], mc["dim"], mc["rot_dim"], mc["vdim"], mc["kv_rank"]
+    rot = dict(mc["rot"])
+    if not use_scaling:
+        rot.pop("scaling", None)
+    freqs, mag = yarn_frequencies(rot)
+    q = (h @ W[pre + "q"].T).reshape(T, H, d + dr)
+    down = h @ W[pre + "dkv"].T
+    c = unit_rms(down[:, :R], eps) * W[pre + "dkv.norm"]
+    kr = np.stack([rotate_halves(down[t, R:], t, freqs, mag) for t in range(T)])
+    kp = (c @ W[pre + "uk"].T).reshape(T, H, d)
+    v = (c @ W[pre + "uv"].T).reshape(T, H, dv)
+    gate = sigmoid(h @ W[pre + "g"].T) if use_gate else np.ones((T, H))
+    out = np.zeros((T, H, dv))
+    for i in range(T):
+        lo = 0 if reach is None else max(0, i - reach + 1)
+        for hd in range(H):
+            qr = rotate_halves(q[i, hd, d:], i, freqs, mag)
+            s = np.array([q[i, hd, :d] @ kp[j, hd] + qr @ kr[j] for j in range(lo, i + 1)]) * mc["scale"]
+            p = np.exp(s - s.max())
+            out[i, hd] = (p / p.sum()) @ v[lo:i + 1, hd] * gate[i, hd]
+    return out.reshape(T, H * dv) @ W[pre + "o"].T
+
+
+def relu_gated_feed_forward(W, pre, h):
+    gate = np.maximum(h @ W[pre + "gate"].T + W[pre + "gate.b"], 0.0)
+    return (gate * (h @ W[pre + "up"].T + W[pre + "up.b"])) @ W[pre + "down"].T + W[pre + "down.b"]
+
+
+def squared_relu_expert(W, pre, a):
+    return (np.maximum(a @ W[pre + "up"].T, 0.0) ** 2) @ W[pre + "down"].T
+
+
+def grouped_choice(s, correction, router, use_correction=True, use_groups=True):
+    """Which of the router's outputs one token uses: scores plus the correction decide, only inside the `keep` groups of neighbours whose best such
+    score is largest.  -> chosen indices (largest first)."""
+    n = len(s)
+    choice = s + (correction if use_correction else 0.0)
+    gr = router.get("groups")
+    if gr and use_groups:
+        size = n // gr["count"]
+        best = np.array([choice[g * size:(g + 1) * size].max() for g in range(gr["count"])])
+        kept = np.argsort(-best, kind="stable")[:gr["keep"]]
+        masked = np.full(n, -np.inf)
+        for g in kept:
+            masked[g * size:(g + 1) * size] = choice[g * size:(g + 1) * size]
+        choice = masked
+    return [int(e) for e in np.argsort(-choice, kind="stable")[:router["top"]]]
+
+
+def routed_experts(W, pre, h, mlp, use_identity=True, use_shared=True, **choice_kw):
+    """Soft-max router over experts + identity experts; the chosen ones' soft-max scores (as they are) weigh their outputs; an identity expert hands
+    its input on; a shared expert runs for every token."""
+    r = mlp["router"]
+    E, ident = r["experts"], r.get("identity", 0)
+    out = np.zeros_like(h)
+    for t in range(h.shape[0]):
+        z = W[pre + "router"] @ h[t]
+        s = np.exp(z - z.max())
+        s /= s.sum()
+        for e in grouped_choice(s, W[pre + "correction"] if pre + "correction" in W else 0.0, r, **choice_kw):
+            if e < E:
+                out[t] += s[e] * squared_relu_expert(W, f"{pre}e{e}.", h[t])
+            elif use_identity:
+                out[t] += s[e] * h[t]
+    if mlp.get("shared") and use_shared:
+        out += squared_relu_expert(W, pre + "shared.", h)
+    return out
+
+
+def run_pokatar(cfg, W, tokens, per_layer=None, attn_kw=None, latent_kw=None, moe_kw=None):
+    """-> logits [T, vocab]; per_layer (a list) receives the residual stream after every layer."""
+    eps = cfg["norm"]["eps"]
+    x = W["embed"][np.asarray(tokens)].astype(np.float64)
+    for i, lc in enumerate(cfg["layers"]):
+        p = f"l{i}."
+        h = centred_norm(x, W[p + "norm1"], eps)
+        if lc["type"] == "attention":
+            x = x + sink_gated_attention(W, p + "mix.", h, lc["mixer"], eps, **(attn_kw or {}))
+        elif lc["type"] == "latent_attention":
+            x = x + shared_key_latent_attention(W, p + "mix.", h, lc["mixer"], eps, **(latent_kw or {}))
+        else:
+            raise ValueError(lc["type"])
+        mlp = lc.get("mlp")
+        if mlp:
+            h = centred_norm(x, W[p + "norm2"], eps)
+            if mlp["kind"] == "dense":
+                x = x + relu_gated_feed_forward(W, p + "mlp.", h)
+            else:
+                x = x + routed_experts(W, p + "mlp.", h, mlp, **(moe_kw or {}))
+        if per_layer is not None:
+            per_layer.append(x.copy())
+    return centred_norm(x, W["final.norm"], eps) @ W["embed"].T
