@@ -56,7 +56,8 @@ def parse():
                     "matrices; powerserve_amd/bench_seq.py SIZES, comma-separated, or 'all'): the sizes 2048x6 / 4096x3 beside the Q4_K Llama path at equal width, "
                     "the sizes v2048x6 / v4096x3 (parallel layers, windowed attention with pooled blocks beside gated linear attention) beside the layer-list model of equal size, "
                     "the sizes z2048x6 / z4096x3 (Zusolix: depth-averaged parallel layers, soft-capped causal attention or a gated recurrence, mixture-of-experts feed-forwards) "
-                    "beside the v sizes")
+                    "beside the v sizes, the sizes p2048x6 / p4096x3 (Pokatar: pre-norm layers, sink attention or shared-key latent attention, relu-gated dense and "
+                    "squared-relu expert feed-forwards) beside the z sizes")
     ap.add_argument("--layer-list-portion", type=int, default=512, help="--layer-list: tokens per launch sequence of the prefill")
     ap.add_argument("--prefill-warmup-tokens", type=int, default=128, help="untimed tokens forwarded before the timed prefill (first use of the prefill kernels in the process; 0: none)")
     ap.add_argument("--wide-chunk", type=int, default=512, help="side leg: prefill in chunks of this many tokens (0: skip)")

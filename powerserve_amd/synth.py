@@ -354,11 +354,91 @@ def _zusolix_tensors(cfg: dict, seed: int) -> dict:
     return t
 
 
+def pokatar_attention(heads: int, kv_heads: int, dim: int, vdim: int, scale: float) -> dict:
+    """mixer entry of a Pokatar attention layer"""
+    return {"heads": int(heads), "kv_heads": int(kv_heads), "dim": int(dim), "vdim": int(vdim), "scale": float(scale)}
+
+
+def pokatar_latent(heads: int, dim: int, rot_dim: int, vdim: int, kv_rank: int, scale: float, base: float = 10000.0, scaling: tuple | None = None) -> dict:
+    """mixer entry of a Pokatar latent-attention layer; scaling: (factor, original, fast, slow) or None"""
+    rot = {"base": float(base), "dims": int(rot_dim)}
+    if scaling:
+        rot["scaling"] = {"factor": float(scaling[0]), "original": int(scaling[1]), "fast": float(scaling[2]), "slow": float(scaling[3])}
+    return {"heads": int(heads), "dim": int(dim), "rot_dim": int(rot_dim), "vdim": int(vdim), "kv_rank": int(kv_rank), "scale": float(scale), "rot": rot}
+
+
+def pokatar_layer(kind: str, mixer: dict, ff: int | None = None, moe: tuple | None = None, shared: int | None = None) -> dict:
+    """One entry of a Pokatar configuration's 'layers'.  kind 'attention' / 'latent_attention'; the feed-forward is dense (ff), a mixture
+    (moe = (experts, top, expert ff, identity experts, groups, groups kept) -- groups 0: no group limit; shared = the shared expert's ff or None), or absent."""
+    mlp = None
+    if moe:
+        experts, top, eff, identity, groups, keep = moe
+        router = {"experts": int(experts), "top": int(top), "identity": int(identity)}
+        if groups:
+            router["groups"] = {"count": int(groups), "keep": int(keep)}
+        mlp = {"kind": "moe", "router": router, "expert": {"ff": int(eff)}}
+        if shared:
+            mlp["shared"] = {"ff": int(shared)}
+    elif ff:
+        mlp = {"kind": "dense", "ff": int(ff)}
+    return {"type": kind, "mixer": dict(mixer), "mlp": mlp}
+
+
+def pokatar_config(width: int, vocab: int, layers: list, eps: float = 1e-5) -> dict:
+    return {"architecture": "Pokatar", "layers": layers, "norm": {"eps": float(eps)}, "vocab": int(vocab), "width": int(width)}
+
+
+def _pokatar_tensors(cfg: dict, seed: int) -> dict:
+    rng = np.random.default_rng(seed)
+    W = cfg["width"]
+
+    def lin(n, k, gain=1.0):
+        return rng.standard_normal((n, k), dtype=np.float32) * np.float32(gain / np.sqrt(k))
+
+    def vec(n, std=0.1, mean=0.0):
+        return (rng.standard_normal(n, dtype=np.float32) * np.float32(std) + np.float32(mean)).astype(np.float32)
+
+    t = {"embed": rng.standard_normal((cfg["vocab"], W), dtype=np.float32)}
+    for i, lc in enumerate(cfg["layers"]):
+        p, m, mc = f"l{i}.", f"l{i}.mix.", lc["mixer"]
+        t[p + "norm1"] = vec(W, 0.2, 1.0)
+        H, d, dv = mc["heads"], mc["dim"], mc["vdim"]
+        if lc["type"] == "attention":
+            G = mc["kv_heads"]
+            t[m + "q"], t[m + "k"], t[m + "v"], t[m + "g"] = lin(H * d, W), lin(G * d, W), lin(G * dv, W), lin(H * dv, W, 2.0)
+            t[m + "q.norm"], t[m + "k.norm"] = vec(d, 0.3, 1.0), vec(d, 0.3, 1.0)
+        elif lc["type"] == "latent_attention":
+            R, dr = mc["kv_rank"], mc["rot_dim"]
+            t[m + "q"], t[m + "dkv"], t[m + "dkv.norm"] = lin(H * (d + dr), W, 1.5), lin(R + dr, W, 1.5), vec(R, 0.3, 1.0)
+            t[m + "uk"], t[m + "uv"], t[m + "g"] = lin(H * d, R, 1.5), lin(H * dv, R), lin(H, W, 2.0)
+        else:
+            raise ValueError(lc["type"])
+        t[m + "o"] = lin(W, H * dv)
+        mlp = lc.get("mlp")
+        if mlp:
+            t[p + "norm2"] = vec(W, 0.2, 1.0)
+            q = p + "mlp."
+            if mlp["kind"] == "dense":
+                ff = mlp["ff"]
+                t[q + "gate"], t[q + "up"], t[q + "down"] = lin(ff, W), lin(ff, W), lin(W, ff)
+                t[q + "gate.b"], t[q + "up.b"], t[q + "down.b"] = vec(ff, 0.3), vec(ff, 0.3), vec(W, 0.3)
+            else:
+                r, ff = mlp["router"], mlp["expert"]["ff"]
+                for e in range(r["experts"]):
+                    t[f"{q}e{e}.up"], t[f"{q}e{e}.down"] = lin(ff, W, 1.5), lin(W, ff)
+                rows = r["experts"] + r.get("identity", 0)
+                t[q + "router"], t[q + "correction"] = lin(rows, W, 2.0), vec(rows, 0.5 / rows)
+                if mlp.get("shared"):
+                    t[q + "shared.up"], t[q + "shared.down"] = lin(mlp["shared"]["ff"], W, 1.5), lin(W, mlp["shared"]["ff"])
+    t["final.norm"] = vec(W, 0.2, 1.0)
+    return t
+
+
 def seq_tensors(cfg: dict, seed: int = 0, decay_rank: int = 8) -> dict:
     """Random-init tensors of a layer-list configuration, name -> float32 array already rounded to bfloat16 (what the file will hold)."""
     from .safetensors_io import f32_to_bf16_bits
-    if cfg.get("architecture") in ("Vobisun", "Zusolix"):
-        t = _parallel_tensors(cfg, seed, decay_rank) if cfg["architecture"] == "Vobisun" else _zusolix_tensors(cfg, seed)
+    if cfg.get("architecture") in ("Vobisun", "Zusolix", "Pokatar"):
+        t = {"Vobisun": lambda: _parallel_tensors(cfg, seed, decay_rank), "Zusolix": lambda: _zusolix_tensors(cfg, seed), "Pokatar": lambda: _pokatar_tensors(cfg, seed)}[cfg["architecture"]]()
         return {k: (f32_to_bf16_bits(v).astype(np.uint32) << 16).view(np.float32).reshape(v.shape) for k, v in t.items()}
     rng = np.random.default_rng(seed)
     W, taps = cfg["width"], cfg["canon"]["taps"]

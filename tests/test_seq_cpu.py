@@ -91,7 +91,9 @@ def test_ctypes_descriptors_match_the_header(tmp_path):
                    'offsetof(ps_seq_layer, beside), offsetof(ps_seq_layer, in_bias), offsetof(ps_seq_layer, tau), offsetof(ps_seq_desc, embed_scale), '
                    'offsetof(ps_seq_desc, max_context));'
                    'printf("%zu %zu %zu %zu %zu %zu %zu\\n", offsetof(ps_seq_layer, res_scale), offsetof(ps_seq_layer, depth_mix), offsetof(ps_seq_layer, softcap), '
-                   'offsetof(ps_seq_layer, qtemp_every), offsetof(ps_seq_layer, experts), offsetof(ps_seq_layer, shared_down), offsetof(ps_seq_desc, norm_groups));return 0;}\n')
+                   'offsetof(ps_seq_layer, qtemp_every), offsetof(ps_seq_layer, experts), offsetof(ps_seq_layer, shared_down), offsetof(ps_seq_desc, norm_groups));'
+                   'printf("%zu %zu %zu %zu %zu %zu %zu\\n", offsetof(ps_seq_layer, head_norm), offsetof(ps_seq_layer, yarn_factor), offsetof(ps_seq_layer, yarn_original), '
+                   'offsetof(ps_seq_layer, ff_up_bias), offsetof(ps_seq_layer, moe_identity), offsetof(ps_seq_layer, moe_correction), offsetof(ps_seq_desc, norm_center));return 0;}\n')
     exe = str(tmp_path / "sz")
     subprocess.run(["gcc", "-I" + os.path.join(ROOT, "include"), str(src), "-o", exe], check=True)
     got = [int(x) for x in subprocess.run([exe], check=True, capture_output=True, text=True).stdout.split()]
@@ -99,7 +101,9 @@ def test_ctypes_descriptors_match_the_header(tmp_path):
                    hip.SeqDesc.layers.offset, hip.SeqLayer.beside.offset, hip.SeqLayer.in_bias.offset, hip.SeqLayer.tau.offset, hip.SeqDesc.embed_scale.offset,
                    hip.SeqDesc.max_context.offset,
                    hip.SeqLayer.res_scale.offset, hip.SeqLayer.depth_mix.offset, hip.SeqLayer.softcap.offset, hip.SeqLayer.qtemp_every.offset, hip.SeqLayer.experts.offset,
-                   hip.SeqLayer.shared_down.offset, hip.SeqDesc.norm_groups.offset]
+                   hip.SeqLayer.shared_down.offset, hip.SeqDesc.norm_groups.offset,
+                   hip.SeqLayer.head_norm.offset, hip.SeqLayer.yarn_factor.offset, hip.SeqLayer.yarn_original.offset, hip.SeqLayer.ff_up_bias.offset,
+                   hip.SeqLayer.moe_identity.offset, hip.SeqLayer.moe_correction.offset, hip.SeqDesc.norm_center.offset]
 
 
 def test_plain_statement_is_causal_and_windowed():
@@ -261,6 +265,105 @@ def test_plain_zusolix_statement_reach_and_pieces():
         s = seq_oracle.sigmoid(W["l0.mlp.router"] @ h[i])
         keep = np.argsort(-s)[:2]
         assert np.allclose(full[i], sum(seq_oracle.one_expert(W, "l0.mlp.e%d." % e, s[e] * h[i]) for e in keep))
+
+
+KCFG = synth.pokatar_config(24, 30, [
+    synth.pokatar_layer("attention", synth.pokatar_attention(4, 2, 6, 10, 0.25), moe=(3, 2, 8, 2, 5, 2), shared=5),
+    synth.pokatar_layer("latent_attention", synth.pokatar_latent(3, 6, 4, 5, 7, 0.3, 77.0, (3.0, 40, 8.0, 0.5)), ff=20),
+    synth.pokatar_layer("latent_attention", synth.pokatar_latent(2, 4, 6, 4, 9, 0.5, 9.0))], eps=1e-5)
+
+
+def test_pokatar_configuration_maps_onto_layer_descriptors(tmp_path):
+    t = synth.write_seq_model_dir(str(tmp_path), KCFG, 1)
+    cfg = seqmodel.read_config(str(tmp_path))
+    up = FakeUp()
+    st = safetensors_io.SafeTensors(str(tmp_path / "model.safetensors"))
+    layers, top = seqmodel.ARCHITECTURES[cfg["architecture"]](cfg, st, up)
+    bits = safetensors_io.f32_to_bf16_bits
+    assert (top["width"], top["vocab"], top["canon_taps"], top["norm_offset"], top["norm_center"], top["logit_scale"]) == (24, 30, 1, 0.0, 1, 1.0)
+    assert top["head"] == top["embed"]  # the logits are taken against the embedding table
+    a, b, c = layers
+    assert all(x.form == seqmodel.LAYER_PRENORM and x.canon1 is None and x.norm1b is None and x.depth_mix is None for x in layers)
+    # attention: q | k | v | g stacked, a gate row per output element, norms per head with [dim] weights, unit values, a sink of zeros
+    assert (a.kind, a.heads, a.kv_heads, a.dim, a.vdim, a.window, a.pool, a.rot_dims, a.gated, a.head_norm, a.v_unit) == (seqmodel.MIX_WINATTN, 4, 2, 6, 10, 0, 0, 0, 2, 1, 1)
+    assert up.mats[a.in_cat - 1001].shape == (24 + 12 + 20 + 40, 24) and np.array_equal(up.mats[a.in_cat - 1001][56:], bits(t["l0.mix.g"]))
+    assert up.vecs[a.qnorm - 1].shape == (6,) and up.vecs[a.knorm - 1].shape == (6,) and not up.vecs[a.sink - 1].any() and up.vecs[a.sink - 1].shape == (4,) and a.in_bias is None
+    # latent attention: q | dkv | g stacked, no query latent, everything before the token, the scaling constants
+    assert (b.kind, b.heads, b.dim, b.vdim, b.q_rank, b.kv_rank, b.rot_dim, b.rot_dims, b.window, b.gated) == (seqmodel.MIX_LATENT, 3, 6, 5, 0, 7, 4, 4, 0, 1)
+    assert (b.yarn_factor, b.yarn_original, b.yarn_fast, b.yarn_slow, b.rot_base) == (3.0, 40, 8.0, 0.5, 77.0) and (c.yarn_factor, c.yarn_original) == (0.0, 0)
+    assert np.array_equal(up.mats[b.in_cat - 1001], np.concatenate([bits(t["l1.mix." + n]) for n in ("q", "dkv", "g")])) and up.mats[b.in_cat - 1001].shape == (30 + 11 + 3, 24)
+    assert np.array_equal(up.mats[b.ukv - 1001], np.concatenate([bits(t["l1.mix.uk"]), bits(t["l1.mix.uv"])])) and b.uq is None and b.qnorm is None
+    # the dense feed-forward: gate / up rows alternating, their biases alike, a bias on the way down
+    assert (b.ff_kind, b.ff, c.ff_kind) == (seqmodel.FF_DENSE_RELU_GLU, 20, seqmodel.FF_NONE)
+    ub = up.vecs[b.ff_up_bias - 1]
+    assert ub.shape == (40,) and np.array_equal(ub[0::2], t["l1.mlp.gate.b"]) and np.array_equal(ub[1::2], t["l1.mlp.up.b"]) and np.array_equal(up.vecs[b.ff_down_bias - 1], t["l1.mlp.down.b"])
+    assert np.array_equal(up.mats[b.ff_up - 1001][1::2], bits(t["l1.mlp.up"]))
+    # the experts: one matrix each way; the router has rows for the identity experts too; groups over all of them
+    assert (a.ff_kind, a.ff, a.experts, a.top, a.shared_ff, a.moe_identity, a.moe_softmax, a.moe_groups, a.moe_keep, a.moe_weight_output) == (seqmodel.FF_MOE_RELU2, 8, 3, 2, 5, 2, 1, 5, 2, 1)
+    assert up.mats[a.ff_up - 1001].shape == (3 * 8, 24) and up.mats[a.ff_down - 1001].shape == (3 * 24, 8) and np.array_equal(up.mats[a.ff_up - 1001][8:16], bits(t["l0.mlp.e1.up"]))
+    assert up.vecs[a.router - 1].shape == (5, 24) and up.vecs[a.moe_correction - 1].shape == (5,) and up.mats[a.shared_up - 1001].shape == (5, 24) and a.shared_gate is None
+    # what the file and the configuration do not have does not exist
+    less = {n: st.f32(n) for n in st.names() if not n.endswith((".b", "correction", ".g", "q.norm"))}
+    cfg2 = json.loads(json.dumps(KCFG))
+    del cfg2["layers"][0]["mlp"]["router"]["groups"], cfg2["layers"][0]["mlp"]["router"]["identity"], cfg2["layers"][0]["mlp"]["shared"], cfg2["layers"][1]["mixer"]["rot"]["scaling"]
+    less["l0.mlp.router"] = less["l0.mlp.router"][:3]
+    synth.write_seq_model_dir(str(tmp_path / "less"), cfg2, 1, tensors=less)
+    layers, _ = seqmodel.ARCHITECTURES["Pokatar"](cfg2, safetensors_io.SafeTensors(str(tmp_path / "less" / "model.safetensors")), FakeUp())
+    a, b, _ = layers
+    assert (a.gated, b.gated, a.qnorm, a.moe_correction, a.moe_groups, a.moe_identity, a.shared_up, b.ff_up_bias, b.ff_down_bias, b.yarn_factor) == (0, 0, None, None, 0, 0, None, None, None, 0.0)
+    assert a.knorm is not None
+    for key, val in (("type", "conveyor"), ("mlp", {"kind": "sparse", "ff": 8})):
+        bad = json.loads(json.dumps(KCFG))
+        bad["layers"][1][key] = val
+        with pytest.raises(seqmodel.ConfigError):
+            seqmodel.ARCHITECTURES["Pokatar"](bad, st, FakeUp())
+    for key, val in (("top", 6), ("groups", {"count": 2, "keep": 1}), ("groups", {"count": 5, "keep": 1})):  # more than the router has; groups that do not divide; top beyond what stays
+        bad = json.loads(json.dumps(KCFG))
+        bad["layers"][0]["mlp"]["router"][key] = val
+        with pytest.raises(seqmodel.ConfigError):
+            seqmodel.ARCHITECTURES["Pokatar"](bad, st, FakeUp())
+
+
+def test_plain_pokatar_statement_reach_and_pieces():
+    """causal, and every later token sees a changed one; the layer norm ignores a shift; the sink takes its share; the frequency ramp ends where it should; the
+    router's choice stays inside the best groups and an identity expert hands its input on"""
+    t = synth.seq_tensors(KCFG, 2)
+    rng = np.random.default_rng(0)
+    a = rng.integers(0, 30, 20)
+    b = a.copy()
+    b[6] = (b[6] + 1) % 30
+    la, lb = seq_oracle.run_pokatar(KCFG, t, a), seq_oracle.run_pokatar(KCFG, t, b)
+    assert np.array_equal(la[:6], lb[:6]) and min(np.abs(la[i] - lb[i]).max() for i in range(6, 20)) > 1e-6
+    x = rng.standard_normal((4, 12))
+    assert np.abs(seq_oracle.centred_norm(x, np.ones(12), 0.0) - seq_oracle.centred_norm(x + 5.0, np.ones(12), 0.0)).max() < 1e-12
+    assert abs(np.mean(seq_oracle.centred_norm(x, np.ones(12), 1e-5))) < 1e-12
+    p = seq_oracle.sink_softmax(np.array([0.0, 0.0, 0.0]))
+    assert np.allclose(p, 0.25) and np.allclose(seq_oracle.sink_softmax(np.array([50.0])), 1.0) and np.allclose(seq_oracle.sink_softmax(np.array([-50.0])), 0.0, atol=1e-20)
+    # base 100, 8 dims: f = 1, 100^-1/4, 100^-1/2, 100^-3/4; original 40: pairs turning more than 8 times in 40 positions keep their frequency, fewer than 1/2 are divided
+    f, mag = seq_oracle.yarn_frequencies({"dims": 8, "base": 100.0, "scaling": {"factor": 4.0, "original": 40, "fast": 8.0, "slow": 0.5}})
+    plain = 100.0 ** (-np.arange(4) / 4.0)
+    lo, hi = max(np.floor(8 * np.log(40 / (2 * np.pi * 8.0)) / (2 * np.log(100.0))), 0), min(np.ceil(8 * np.log(40 / (2 * np.pi * 0.5)) / (2 * np.log(100.0))), 7)
+    assert (lo, hi) == (0, 3) and np.allclose(f, plain * (1 - np.arange(4) / 3) + plain / 4 * np.arange(4) / 3) and abs(mag - (0.1 * np.log(4.0) + 1)) < 1e-12
+    assert np.allclose(seq_oracle.yarn_frequencies({"dims": 8, "base": 100.0})[0], plain)
+    v = rng.standard_normal(8)
+    r = seq_oracle.rotate_halves(v, 3, plain, 1.0)
+    assert np.allclose(np.hypot(r[:4], r[4:]), np.hypot(v[:4], v[4:])) and np.allclose(seq_oracle.rotate_halves(v, 0, plain, 1.5), 1.5 * v)
+    # five router rows in five groups of one of which two stay: exactly the two best corrected scores; with one group of five the same two
+    s, corr = np.array([0.1, 0.3, 0.15, 0.25, 0.2]), np.array([0.0, -0.2, 0.0, 0.0, 0.2])
+    assert seq_oracle.grouped_choice(s, corr, {"top": 2, "groups": {"count": 5, "keep": 2}}) == [4, 3]
+    assert seq_oracle.grouped_choice(s, 0.0, {"top": 2}) == [1, 3]
+    # six rows in three pairs, one pair stays: the best single row decides the pair, the second choice is its neighbour however small
+    s6 = np.array([0.05, 0.3, 0.25, 0.2, 0.1, 0.1])
+    assert seq_oracle.grouped_choice(s6, 0.0, {"top": 2, "groups": {"count": 3, "keep": 1}}) == [1, 0]
+    W = {k: np.asarray(v, np.float64) for k, v in t.items()}
+    h = rng.standard_normal((6, 24))
+    mlp = KCFG["layers"][0]["mlp"]
+    full = seq_oracle.routed_experts(W, "l0.mlp.", h, mlp, use_shared=False)
+    for i in range(6):
+        z = W["l0.mlp.router"] @ h[i]
+        sc = np.exp(z) / np.exp(z).sum()
+        keep = np.argsort(-(sc + W["l0.mlp.correction"]))[:2]  # (five groups of one, two stay: the group limit changes nothing here)
+        assert np.allclose(full[i], sum(sc[e] * (seq_oracle.squared_relu_expert(W, "l0.mlp.e%d." % e, h[i]) if e < 3 else h[i]) for e in keep))
 
 
 def test_the_small_library_exports_what_its_models_need():
