@@ -41,6 +41,8 @@ struct dn_args {
     const int32_t *g_sel, *g_seg, *g_list;
     const float *g_scale;
     long long wstride;
+    const float *g_ident, *g_ident_w; // grouped mat-vec: a slot without a matrix adds g_ident_w[slot] * g_ident[row][n] to output n
+    long long g_ident_ld;
 };
 
 // rows of A that exist and where they start (ring rows relative to the step's position)
@@ -315,11 +317,15 @@ __global__ __launch_bounds__(256) void dense_mv_grouped_kernel(dn_args g) {
     const bool vec = (K * (long long)sizeof(WT)) % 16 == 0;
     for (long long nb = ((long long)blockIdx.x * 4 + wave) * RW; nb < g.N; nb += (long long)gridDim.x * 4 * RW) {
         float acc[RW];
+        float ident = 0.f; // the summed weights of the row's slots that have no matrix (identity experts)
 #pragma unroll
         for (int q = 0; q < RW; q++) acc[q] = 0.f;
         for (int c = 0; c < inner; c++) {
             const int sel = g.g_sel[(long long)r * inner + c];
-            if (sel >= g.groups) continue; // (a slot whose choice has no matrix -- an identity expert -- adds nothing here; the same for every lane of the block)
+            if (sel >= g.groups) { // (no product for this slot; the same for every lane of the block)
+                if (g.g_ident) ident += g.g_ident_w[(long long)r * inner + c];
+                continue;
+            }
             const WT *W = (const WT *)g.w + (long long)sel * g.wstride;
             const float *x = xs + (long long)c * Kp;
             if (vec) {
@@ -368,6 +374,11 @@ __global__ __launch_bounds__(256) void dense_mv_grouped_kernel(dn_args g) {
         for (int q = 0; q < RW; q++) {
 #pragma unroll
             for (int o = 32; o > 0; o >>= 1) acc[q] += __shfl_xor(acc[q], o, 64);
+        }
+        if (ident != 0.f && lane == 0) {
+#pragma unroll
+            for (int q = 0; q < RW; q++)
+                if (nb + q < g.N) acc[q] = fmaf(ident, g.g_ident[(long long)r * g.g_ident_ld + nb + q], acc[q]);
         }
 #pragma unroll
         for (int q = 0; q < RW; q++) dn_put(g, r, nb + q, acc[q], acc[RW > 1 ? (q ^ 1) : q], lane == 0 && nb + q < g.N);
@@ -491,6 +502,7 @@ int psk_dense(hipStream_t st, const psk_dense_args &a) {
     g.N = a.w->N; g.K = a.w->K; g.out = a.out; g.ldo = a.ldo; g.bias = a.bias; g.act = a.act; g.act_p = a.act_p; g.act_q = a.act_q;
     g.alpha = a.alpha; g.mu = a.mu; g.shift0 = a.shift0; g.accum = a.accum; g.out_scale = a.out_scale;
     g.groups = 0; g.g_adiv = 1; g.g_odiv = 1; g.g_inner = 1; g.g_sel = nullptr; g.g_seg = nullptr; g.g_list = nullptr; g.g_scale = nullptr; g.wstride = 0;
+    g.g_ident = a.g_ident; g.g_ident_w = a.g_ident_w; g.g_ident_ld = a.g_ident_ld;
     const bool bf = a.w->dtype == PS_BF16;
     const size_t kp4 = (size_t)((g.K + 7) / 8 * 8) * 4;
     if (a.groups > 0) {

@@ -44,7 +44,6 @@ __global__ __launch_bounds__(256) void winattn_prep_kernel(const ps_seq_step *st
     const int t = blockIdx.x, tid = threadIdx.x;
     const long long pos = step->pos0 + t;
     const int nq = H * d, nk = G * d, nv = G * dv, half = rot_dims / 2;
-    float *hinv = cs + rot_dims + 2; // per-head norms: 1 / rms of every q head, k head, v head ([H | G | G])
     const float *qt = y + (long long)t * ldy, *kt = qt + nq, *vt = kt + nk;
     float *ring = step->state + ring_off + (pos % cap) * (long long)(nk + nv);
     // a query temperature that grows with the position in steps of qt_every tokens: 1 + coef ln(floor((pos + 1) / every) + 1)
@@ -60,25 +59,14 @@ __global__ __launch_bounds__(256) void winattn_prep_kernel(const ps_seq_step *st
     a = wa_wave_sum(a);
     b = wa_wave_sum(b);
     if ((tid & 63) == 0) { red[tid >> 6] = a; red[4 + (tid >> 6)] = b; }
-    if (head_norm || v_unit) { // a wave per head: heads 0 .. H - 1 of q, then G of k, then G of v
-        for (int hd = tid >> 6; hd < H + 2 * G; hd += 4) {
-            const bool isq = hd < H, isk = !isq && hd < H + G;
-            const float *src = isq ? qt + hd * d : isk ? kt + (hd - H) * d : vt + (hd - H - G) * dv;
-            const int n = isq || isk ? d : dv;
-            const bool on = isq ? (head_norm && qnorm) : isk ? (head_norm && knorm) : v_unit != 0;
-            float ss = 0.f;
-            if (on) for (int i = tid & 63; i < n; i += 64) ss += src[i] * src[i];
-            ss = wa_wave_sum(ss);
-            if ((tid & 63) == 0) hinv[hd] = on ? 1.f / sqrtf(ss / (float)n + eps) : 1.f;
-        }
-    }
     __syncthreads();
     const float ia = qnorm && !head_norm ? 1.f / sqrtf((red[0] + red[1] + red[2] + red[3]) / (float)nq + eps) : 1.f;
     const float ib = knorm && !head_norm ? 1.f / sqrtf((red[4] + red[5] + red[6] + red[7]) / (float)nk + eps) : 1.f;
-    // element i of a projection (c = its index in its head): normed, and where c < rot_dims turned together with its partner
-    auto turned = [&](const float *src, const float *w, float inv, const float *hi, int i) {
+    // element i of a projection (c = its index in its head): normed, and where c < rot_dims turned together with its partner; wc: 1 = one weight vector of d
+    // numbers for every head (indexed by c), 0 = a weight per element of the projection
+    auto turned = [&](const float *src, const float *w, float inv, int i, int wc) {
         const int c = i % d;
-        if (head_norm) { inv = hi[i / d]; if (w) w += c - i; } // (the head's own statistics; one weight vector for every head: w[i] below reads w[c])
+        if (w && wc) w += c - i;
         const float self = src[i] * inv * (w ? w[i] : 1.f);
         if (c >= 2 * half) return self;
         int partner, pair;
@@ -97,13 +85,35 @@ __global__ __launch_bounds__(256) void winattn_prep_kernel(const ps_seq_step *st
         const float sum = (pos == pb * pool ? 0.f : mean[c]) + v;
         mean[c] = pos == pb * pool + pool - 1 ? sum / (float)pool : sum;
     };
+    if (head_norm || v_unit) {
+        // statistics per head: a WAVE per head (the heads of q, then k, then v, dealt over the token's blocks and their waves) sums, norms, turns and stores it
+        const int lane = tid & 63;
+        for (int hd = blockIdx.y * 4 + (tid >> 6); hd < H + 2 * G; hd += 4 * gridDim.y) {
+            const bool isq = hd < H, isk = !isq && hd < H + G;
+            const int n = isq || isk ? d : dv, e0 = isq ? hd * d : isk ? (hd - H) * d : (hd - H - G) * dv; // (e0: the head's first element in its projection)
+            const float *src = isq ? qt : isk ? kt : vt, *w = isq ? qnorm : isk ? knorm : nullptr;
+            const bool own = isq || isk ? head_norm && w : v_unit != 0;
+            float ss = 0.f;
+            if (own) for (int c = lane; c < n; c += 64) ss += src[e0 + c] * src[e0 + c];
+            ss = wa_wave_sum(ss);
+            const float inv = own ? 1.f / sqrtf(ss / (float)n + eps) : isq ? ia : isk ? ib : 1.f;
+            for (int c = lane; c < n; c += 64) {
+                if (isq) { qo[(long long)t * ldq + e0 + c] = turned(qt, qnorm, inv, e0 + c, head_norm) * qtemp; continue; }
+                const float v = isk ? turned(kt, knorm, inv, e0 + c, head_norm) : vt[e0 + c] * inv;
+                const int i = isk ? e0 + c : nk + e0 + c;
+                ring[i] = v;
+                pooled(i, v);
+            }
+        }
+        return;
+    }
     // the elements of q | k | v are spread over the blocks of a token (gridDim.y; every block has made the sums above for itself)
     for (int e = blockIdx.y * 256 + tid; e < nq + nk + nv; e += 256 * gridDim.y) {
         if (e < nq) {
-            qo[(long long)t * ldq + e] = turned(qt, qnorm, ia, hinv, e) * qtemp;
+            qo[(long long)t * ldq + e] = turned(qt, qnorm, ia, e, 0) * qtemp;
         } else {
             const int i = e - nq;
-            const float v = i < nk ? turned(kt, knorm, ib, hinv + H, i) : (v_unit ? vt[i - nk] * hinv[H + G + (i - nk) / dv] : vt[i - nk]);
+            const float v = i < nk ? turned(kt, knorm, ib, i, 0) : vt[i - nk];
             ring[i] = v;
             pooled(i, v);
         }
@@ -129,8 +139,9 @@ void psk_winattn_prep(hipStream_t st, const ps_seq_step *step, int64_t ring_off,
                       const float *knorm, float eps, int H, int G, int d, int dv, int rot_dims, int pairing, const float *freq, int T, float *q, int64_t ldq, float qt_coef,
                       int qt_every, int head_norm, int v_unit) {
     const int total = H * d + G * (d + dv);
-    const int split = T >= 64 ? 1 : std::min(16, (total + 511) / 512); // few tokens: a token's elements over several blocks
-    hipLaunchKernelGGL(winattn_prep_kernel, dim3(T, split), dim3(256), (size_t)(rot_dims + 2 + H + 2 * G) * 4, st, step, (long long)ring_off, cap, (long long)pool_off, pool, y,
+    // few tokens: a token's elements over several blocks; with statistics per head, its heads (four per block)
+    const int split = head_norm || v_unit ? (T >= 64 ? std::min(2, (H + 2 * G + 3) / 4) : std::min(32, (H + 2 * G + 3) / 4)) : T >= 64 ? 1 : std::min(16, (total + 511) / 512);
+    hipLaunchKernelGGL(winattn_prep_kernel, dim3(T, split), dim3(256), (size_t)(rot_dims + 2) * 4, st, step, (long long)ring_off, cap, (long long)pool_off, pool, y,
                        (long long)ldy, qnorm, knorm, eps, H, G, d, dv, rot_dims, pairing, freq, q, (long long)ldq, qt_coef, qt_every, head_norm, v_unit);
     if (pool > 0 && T > 1) {
         const int rs = G * (d + dv);

@@ -55,6 +55,10 @@ struct psk_dense_args {
     int groups = 0, g_adiv = 1, g_odiv = 1, g_inner = 1;
     const int32_t *g_sel = nullptr, *g_seg = nullptr, *g_list = nullptr;
     const float *g_scale = nullptr;
+    // the grouped mat-vec only (an output per row, no activation): a slot whose g_sel is not below `groups` has no matrix -- an identity expert -- and adds
+    // g_ident_w[slot] * g_ident[row][n] to output n of its row instead of a product (g_ident NULL: nothing)
+    const float *g_ident = nullptr, *g_ident_w = nullptr;
+    int64_t g_ident_ld = 0;
 };
 int psk_dense(hipStream_t st, const psk_dense_args &a);
 void psk_dense_widen(hipStream_t st, const uint16_t *bf16, int64_t n, float *out);

@@ -635,7 +635,10 @@ static void seq_layers(ps_hip_seq *m, float *state, int T, int64_t pos0, bool an
         {
             auto g = mm(l.ff_down, m->t4, l.ff, xr, W);
             grouped(g);
-            if (mv) { g.T = T; g.g_inner = top; g.accum = 1; g.alpha = alpha; }
+            if (mv) {
+                g.T = T; g.g_inner = top; g.accum = 1; g.alpha = alpha;
+                if (l.moe_identity) { g.g_ident = in; g.g_ident_ld = W; g.g_ident_w = m->moe_wgt; summed = true; } // (the identity slots' share inside the same launch)
+            }
             else if (top == 1) { g.T = S; g.accum = 1; g.alpha = alpha; }
             else { g.T = S; g.out = m->moe_y; } // (two slots of a token sit in different tiles: per-slot results, summed below)
             psk_dense(st, g);
