@@ -463,7 +463,8 @@ uint64_t ps_hip_seq_weight_bytes_per_token(const ps_hip_seq *m);
 /* Measurement helper (bench.py's per-kernel roofline): a feed-forward matrix product of T tokens replayed `reps` times over every layer
  * that has one (each launch streams its own layer's weights), between HIP events -> microseconds per launch, the weight bytes and the
  * flops of one launch.  which: 0 the up projection (with its activation), 1 the down projection of the dense feed-forwards; 2 / 3 the same two products of
- * the mixture-of-experts layers (grouped launches over the routing of T embedded tokens; bytes: the experts a launch can touch).  T <= 8 runs the mat-vec. */
+ * the mixture-of-experts layers (grouped launches over the routing of T embedded tokens; bytes: the matrices that routing touches, flops: the slots it sends to an
+ * expert that has matrices -- identity experts take neither).  T <= 8 runs the mat-vec. */
 int ps_hip_seq_bench_kernel(ps_hip_seq *m, int which, int T, int reps, double *us_per_launch, double *bytes, double *flops);
 
 #ifdef __cplusplus

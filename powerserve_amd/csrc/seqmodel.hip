@@ -860,9 +860,16 @@ int ps_hip_seq_bench_kernel(ps_hip_seq *m, int which, int T, int reps, double *u
                 if (mv) { g.T = T; g.g_inner = top; g.out = m->y; }
                 else { g.T = S; g.out = top == 1 ? m->y : m->moe_y; }
             }
-            const int used = std::min(P.d.experts, S); // matrices a launch can touch at most
+            // what this routing makes a launch do: the slots that go to an expert with matrices (identity experts take none) and the matrices they touch
+            std::vector<int32_t> sel((size_t)S);
+            PS_CHECK(c, hipMemcpyAsync(sel.data(), m->moe_sel, (size_t)S * 4, hipMemcpyDeviceToHost, c->stream));
+            PS_CHECK(c, hipStreamSynchronize(c->stream));
+            std::vector<char> seen((size_t)P.d.experts, 0);
+            int real = 0, used = 0;
+            for (int32_t e : sel)
+                if (e >= 0 && e < P.d.experts) { real++; if (!seen[e]) { seen[e] = 1; used++; } }
             per_bytes = (double)dense_bytes(g.w) / P.d.experts * used;
-            per_flops = 2.0 * S * (double)(g.w->N / P.d.experts) * (double)g.w->K;
+            per_flops = 2.0 * real * (double)(g.w->N / P.d.experts) * (double)g.w->K;
         } else if (which == 0) {
             g.w = P.d.ff_up; g.a = m->h; g.lda = m->d.width; g.out = m->t4; g.ldo = P.d.ff;
             if (P.d.ff_kind == PS_FF_DENSE_SWIGLU) g.act = PSD_ACT_SILU_PAIR;
