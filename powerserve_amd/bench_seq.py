@@ -29,12 +29,12 @@ SIZES = {
     "z2048x6": dict(design="Zusolix", width=2048, ff=8192, heads=16, kv_heads=4, dim=128, gru=3072, experts=8, top=2, order="aagaag", layers=6, beside="v2048x6"),
     "z4096x3": dict(design="Zusolix", width=4096, ff=14336, heads=32, kv_heads=8, dim=128, gru=6144, experts=8, top=2, order="aga", layers=3, beside="v4096x3"),
     # Pokatar (pre-norm layers with layer norms; causal attention with a sink, per-head norms and an element-wise gate, or latent attention with a shared rotated
-    # key part; the first layer's feed-forward relu-gated dense, the others 8 squared-relu experts + 2 identity experts in 2 groups of which one stays, top 2, plus
+    # key part; the first layer's feed-forward relu-gated dense, the others 8 squared-relu experts + 2 identity experts in 5 groups of which three stay, top 2, plus
     # a shared expert -- two matrices per expert instead of three, so an inner size of 3/2 x ff/4 and 3/2 x ff/2 holds the Zusolix experts' weights) beside the
     # Zusolix model of equal width, feed-forward size, head counts and layers
-    "p2048x6": dict(design="Pokatar", width=2048, ff=8192, heads=16, kv_heads=4, dim=128, kv_rank=512, rot_dim=64, experts=8, identity=2, groups=(2, 1), top=2,
+    "p2048x6": dict(design="Pokatar", width=2048, ff=8192, heads=16, kv_heads=4, dim=128, kv_rank=512, rot_dim=64, experts=8, identity=2, groups=(5, 3), top=2,
                     order="aalaal", layers=6, beside="z2048x6"),
-    "p4096x3": dict(design="Pokatar", width=4096, ff=14336, heads=32, kv_heads=8, dim=128, kv_rank=512, rot_dim=64, experts=8, identity=2, groups=(2, 1), top=2,
+    "p4096x3": dict(design="Pokatar", width=4096, ff=14336, heads=32, kv_heads=8, dim=128, kv_rank=512, rot_dim=64, experts=8, identity=2, groups=(5, 3), top=2,
                     order="ala", layers=3, beside="z4096x3"),
 }
 
@@ -43,7 +43,7 @@ def config(z: dict, vocab: int = 4096) -> dict:
     H, d = z["heads"], z["dim"]
     if z.get("design") == "Pokatar":
         att = synth.pokatar_attention(H, z["kv_heads"], d, d, float(d ** -0.5))
-        lat = synth.pokatar_latent(H, d, z["rot_dim"], d, z["kv_rank"], float((d + z["rot_dim"]) ** -0.5), 1e6, (4.0, 1024, 32.0, 1.0))
+        lat = synth.pokatar_latent(H, d, z["rot_dim"], d, z["kv_rank"], float((d + z["rot_dim"]) ** -0.5), 5e5, (8.0, 4096, 16.0, 2.0))
         layers = []
         for i, k in enumerate(z["order"]):
             mixer = ("attention", att) if k == "a" else ("latent_attention", lat)

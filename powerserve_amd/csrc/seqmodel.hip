@@ -824,12 +824,15 @@ int ps_hip_seq_bench_kernel(ps_hip_seq *m, int which, int T, int reps, double *u
     PS_CHECK(c, hipSetDevice(c->device));
     const bool moe = which >= 2;
     const int64_t W = m->d.width;
-    if (moe) { // tokens 0, 1, 2, ... embedded as the input: a routing as spread as the router's rows make it
+    auto embed_from = [&](int first) { // tokens first, first + 1, ... embedded as the input: a routing as spread as the router's rows make it
         std::vector<int32_t> ids((size_t)T);
-        for (int i = 0; i < T; i++) ids[i] = i % m->d.vocab;
-        PS_CHECK(c, hipMemcpyAsync(m->tokens, ids.data(), (size_t)T * 4, hipMemcpyHostToDevice, c->stream));
+        for (int i = 0; i < T; i++) ids[i] = (first + i) % m->d.vocab;
+        if (hipMemcpyAsync(m->tokens, ids.data(), (size_t)T * 4, hipMemcpyHostToDevice, c->stream) != hipSuccess) return false;
         psk_embed(c->stream, m->d.embed, m->tokens, m->step, T, m->embed_scale, m->h, W);
-        PS_CHECK(c, hipStreamSynchronize(c->stream));
+        return hipStreamSynchronize(c->stream) == hipSuccess;
+    };
+    if (moe) {
+        if (!embed_from(0)) return seq_fail(c, "seq_bench_kernel: embedding");
     } else {
         psk_fill(c->stream, m->h, 0.01f, (int64_t)m->d.max_batch * W);
     }
@@ -845,8 +848,18 @@ int ps_hip_seq_bench_kernel(ps_hip_seq *m, int which, int T, int reps, double *u
             const int top = P.d.top, S = T * top;
             const bool mv = T <= 8;
             const int rows = P.d.experts + P.d.moe_identity;
-            psk_moe_route(c->stream, m->h, W, P.d.router, P.d.shared_gate, rows, top, P.d.moe_norm_top, W, T, m->moe_sel, m->moe_wgt, m->moe_sg, P.d.moe_softmax,
-                          P.d.moe_correction, P.d.moe_groups, P.d.moe_keep);
+            std::vector<int32_t> sel((size_t)S);
+            // (a few tokens: the first run of tokens none of whose choices is an identity expert, so that a mat-vec launch has its full work)
+            for (int first = 0; first < (mv && P.d.moe_identity ? 64 : 1); first++) {
+                if (first && !embed_from(first)) return seq_fail(c, "seq_bench_kernel: embedding");
+                psk_moe_route(c->stream, m->h, W, P.d.router, P.d.shared_gate, rows, top, P.d.moe_norm_top, W, T, m->moe_sel, m->moe_wgt, m->moe_sg, P.d.moe_softmax,
+                              P.d.moe_correction, P.d.moe_groups, P.d.moe_keep);
+                PS_CHECK(c, hipMemcpyAsync(sel.data(), m->moe_sel, (size_t)S * 4, hipMemcpyDeviceToHost, c->stream));
+                PS_CHECK(c, hipStreamSynchronize(c->stream));
+                bool all_real = true;
+                for (int32_t e : sel) all_real = all_real && e < P.d.experts;
+                if (all_real) break;
+            }
             if (!mv) psk_moe_plan(c->stream, m->moe_sel, S, rows, m->moe_seg, m->moe_list);
             g.groups = P.d.experts; g.g_sel = m->moe_sel;
             if (!mv) { g.g_seg = m->moe_seg; g.g_list = m->moe_list; }
@@ -861,9 +874,6 @@ int ps_hip_seq_bench_kernel(ps_hip_seq *m, int which, int T, int reps, double *u
                 else { g.T = S; g.out = top == 1 ? m->y : m->moe_y; }
             }
             // what this routing makes a launch do: the slots that go to an expert with matrices (identity experts take none) and the matrices they touch
-            std::vector<int32_t> sel((size_t)S);
-            PS_CHECK(c, hipMemcpyAsync(sel.data(), m->moe_sel, (size_t)S * 4, hipMemcpyDeviceToHost, c->stream));
-            PS_CHECK(c, hipStreamSynchronize(c->stream));
             std::vector<char> seen((size_t)P.d.experts, 0);
             int real = 0, used = 0;
             for (int32_t e : sel)

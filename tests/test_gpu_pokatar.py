@@ -24,7 +24,7 @@ CONFIGS = {
                        PL("latent_attention", PLA(2, 5, 4, 9, 10, 0.3, 50.0), moe=(5, 3, 8, 1, 3, 2))], eps=1e-5),
     # sizes the matrix-core kernels take (wide mat-mul: inputs that are multiples of 64; absorbed single-token latent step), top 1, top == what the groups leave,
     # no identity experts, one group
-    "aligned": PC(128, 96, [PL("latent_attention", PLA(4, 32, 16, 16, 64, 0.15, 10000.0, (4.0, 128, 16.0, 2.0)), moe=(8, 1, 64, 0, 2, 1), shared=64),
+    "aligned": PC(128, 96, [PL("latent_attention", PLA(4, 48, 32, 16, 48, 0.15, 10000.0, (4.0, 128, 16.0, 2.0)), moe=(8, 1, 64, 0, 2, 1), shared=64),
                             PL("attention", PA(4, 2, 32, 16, 0.2), ff=192),
                             PL("attention", PA(8, 2, 16, 32, 0.25), moe=(6, 3, 64, 2, 4, 2)),
                             PL("latent_attention", PLA(2, 16, 32, 64, 32, 0.2, 500000.0, (8.0, 64, 32.0, 1.0)), moe=(4, 2, 128, 0, 1, 1))], eps=1e-6),
